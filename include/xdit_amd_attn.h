@@ -1,0 +1,160 @@
+/*
+ * xdit_amd_attn.h — C ABI of the MI355X (gfx950) attention hot path.
+ *
+ * One shared library (libxdit_amd_attn.so) exports the entry points below.  They are what a
+ * foreign-function binding (ctypes, cffi, pybind, a C++ torch op) of xDiT's attention path would
+ * bind on one GPU.  Every pointer is a DEVICE pointer owned by the caller; the library allocates
+ * nothing, keeps nothing after return, never synchronises the device and launches on the stream
+ * the caller passes.  All strides are in ELEMENTS of the tensor's own dtype.  The innermost
+ * (head_dim) stride of every tensor is 1.
+ *
+ * Return value: 0 on success, a negative xdit_status otherwise; the message of the last failure
+ * on the calling thread is available from xdit_attn_last_error().
+ *
+ * Reference interfaces replaced (paths relative to the xDiT source tree):
+ *   - the `(out, lse)` vendor flash-attention forward reached by the backend registry entries
+ *     xfuser/core/distributed/attention_backend.py:504-516 (SDPA_FLASH), :534-548 (SDPA_EFFICIENT),
+ *     :774-823 (AITER), :887-918 (FLASH), and by the per-step kernel call of the legacy ring loop
+ *     xfuser/core/long_ctx_attention/ring/ring_flash_attn.py:105-134            -> xdit_attn_fwd
+ *   - the fp8 forward with per-(batch,head) descales, attention_backend.py:617-642 (FLASH_3_FP8)
+ *     and :717-772 (AITER_FP8)                                                   -> xdit_attn_fwd (dtype FP8)
+ *   - the ring online-softmax merge `update_out_and_lse` called at
+ *     ring_flash_attn.py:138 (+ epilogue :145-148) and torch's `_SDPAMerger._merge_one`
+ *     (torch/distributed/tensor/experimental/_context_parallel/_attention.py:181-182)
+ *                                                                                -> xdit_lse_merge
+ *   - `per_tensor_quant`, attention_backend.py:606-615                           -> xdit_fp8_quant
+ */
+#ifndef XDIT_AMD_ATTN_H
+#define XDIT_AMD_ATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XDIT_ATTN_ABI_VERSION 1
+
+typedef enum {
+  XDIT_OK = 0,
+  XDIT_ERR_INVALID_ARG = -1,   /* null pointer, bad shape/stride/alignment, unsupported option */
+  XDIT_ERR_UNSUPPORTED = -2,   /* a combination this library does not implement (e.g. causal)  */
+  XDIT_ERR_LAUNCH = -3         /* the HIP runtime rejected the launch                          */
+} xdit_status;
+
+typedef enum {
+  XDIT_DTYPE_BF16 = 0,
+  XDIT_DTYPE_FP16 = 1,
+  XDIT_DTYPE_FP32 = 2,
+  XDIT_DTYPE_FP8_E4M3FN = 3    /* OCP e4m3fn (max 448), the fp8 format of gfx950 */
+} xdit_dtype;
+
+/* Logical tensor (B, H, S, D) with arbitrary B/H/S element strides; D stride is 1.
+ * BHSD-contiguous:                stride = {H*S*D, S*D, D}
+ * BSHD-contiguous viewed as BHSD: stride = {S*H*D, D, H*D}                                   */
+typedef struct {
+  int64_t b, h, s;
+} xdit_strides;
+
+/*
+ * Non-causal scaled-dot-product attention forward returning the output and the per-row
+ * log-sum-exp (natural log, softmax scale included):
+ *     s_ij = softmax_scale * sum_d q_id k_jd ,  j over Sk keys of (k,v) then Sk2 keys of (k2,v2)
+ *     out_i = sum_j softmax_j(s_ij) v_j ,  lse_i = log sum_j exp(s_ij)
+ * For FP8 inputs q,k,v are multiplied by q_descale[b,h], k_descale[b,h], v_descale[b,h] first.
+ * Replaces: attention_backend.py:504-516/:774-823/:887-918 (+ :617-642, :717-772 for fp8) and the
+ * kernel call at ring_flash_attn.py:123-134.  The optional second KV segment replaces the
+ * torch.cat of joint (text) keys/values at usp.py:239-241 / ring_flash_attn.py:89-100.
+ */
+typedef struct {
+  uint32_t struct_size;        /* = sizeof(xdit_attn_args) */
+  int32_t dtype;               /* xdit_dtype of q, k, v, k2, v2 */
+  int32_t out_dtype;           /* xdit_dtype of out: same as dtype for bf16/fp16/fp32; bf16 or fp16 for fp8 */
+  int32_t causal;              /* must be 0 */
+  int32_t B, H, D;             /* batch, heads (Hq == Hk), head_dim */
+  int32_t reserved0;
+  int64_t Sq, Sk, Sk2;         /* query rows; keys in segment 1; keys in segment 2 (0 = none) */
+  float softmax_scale;         /* > 0 */
+  float reserved1;
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* k2;              /* may be NULL when Sk2 == 0 */
+  const void* v2;
+  void* out;                   /* (B,H,Sq,D) out_dtype */
+  float* lse;                  /* (B,H,Sq) fp32, may be NULL */
+  xdit_strides q_stride, k_stride, v_stride, k2_stride, v2_stride, out_stride;
+  int64_t lse_stride_b, lse_stride_h;   /* lse stride over Sq is 1 */
+  const float* q_descale;      /* FP8 only: (B,H) fp32 each; NULL means 1.0 */
+  const float* k_descale;
+  const float* v_descale;
+  int64_t descale_stride_b, descale_stride_h;
+  void* stream;                /* hipStream_t; NULL = the null stream */
+} xdit_attn_args;
+
+int xdit_attn_fwd(const xdit_attn_args* args);
+
+/*
+ * One fold of the ring online-softmax merge, in fp32:
+ *     acc_out <- acc_out - sigmoid(block_lse - acc_lse) * (acc_out - block_out)
+ *     acc_lse <- acc_lse - logsigmoid(acc_lse - block_lse)
+ * `first != 0` initialises instead: acc_out <- float(block_out), acc_lse <- block_lse.
+ * If final_out != NULL the merged row is also written there in final_dtype (the epilogue cast
+ * `out.to(q.dtype)`).  acc_out/block_out/final_out are logical (B,H,S,D); acc_lse/block_lse are
+ * logical (B,H,S) with their own B/H/S strides, so the (B,S,H,1) accumulator layout of the legacy
+ * ring and the (B,H,S) layout a kernel returns both map without copies.
+ * Replaces: update_out_and_lse at ring_flash_attn.py:138, the epilogue at :145, and
+ * torch _SDPAMerger._merge_one (…/_context_parallel/_attention.py:161-163, :181-182).
+ */
+typedef struct {
+  uint32_t struct_size;        /* = sizeof(xdit_merge_args) */
+  int32_t block_dtype;         /* xdit_dtype of block_out: bf16, fp16 or fp32 */
+  int32_t final_dtype;         /* xdit_dtype of final_out (ignored when final_out == NULL) */
+  int32_t first;               /* != 0: initialise the accumulator from the block */
+  int32_t B, H, D;
+  int32_t reserved0;
+  int64_t S;
+  float* acc_out;              /* fp32 */
+  float* acc_lse;              /* fp32 */
+  const void* block_out;
+  const float* block_lse;      /* fp32 */
+  void* final_out;             /* may be NULL */
+  xdit_strides acc_out_stride, block_out_stride, final_out_stride;
+  xdit_strides acc_lse_stride, block_lse_stride;
+  void* stream;
+} xdit_merge_args;
+
+int xdit_lse_merge(const xdit_merge_args* args);
+
+/*
+ * Per-(batch,head) abs-max fp8 quantiser: for every (b,h), scale = absmax(x[b,h]) / 448 (or the
+ * value 1.0 if the slice is all zero), y = fp8_e4m3fn(x / scale), descale[b,h] = scale.
+ * `per_tensor != 0` uses one abs-max over the whole tensor and broadcasts it to (B,H), which is
+ * the reference's per_tensor_quant (attention_backend.py:606-615).
+ * `workspace` must hold at least B*H floats... it is the descale output itself; no extra memory.
+ */
+typedef struct {
+  uint32_t struct_size;        /* = sizeof(xdit_quant_args) */
+  int32_t in_dtype;            /* bf16, fp16 or fp32 */
+  int32_t per_tensor;
+  int32_t B, H, D;
+  int64_t S;
+  const void* x;               /* (B,H,S,D) in_dtype */
+  void* y;                     /* (B,H,S,D) fp8 e4m3fn bytes */
+  float* descale;              /* (B,H) fp32, contiguous */
+  xdit_strides x_stride, y_stride;
+  void* stream;
+} xdit_quant_args;
+
+int xdit_fp8_quant(const xdit_quant_args* args);
+
+/* Message of the last error on the calling thread ("" if none). Never NULL. */
+const char* xdit_attn_last_error(void);
+
+/* XDIT_ATTN_ABI_VERSION the library was built with. */
+int xdit_attn_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XDIT_AMD_ATTN_H */

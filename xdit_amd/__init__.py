@@ -1,0 +1,3 @@
+"""MI355X-native attention hot path (joint-attention forward + ring LSE merge) behind
+xDiT's attention call surfaces."""
+from .ops import attn_fwd, lse_merge  # noqa: F401

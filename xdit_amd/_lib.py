@@ -1,0 +1,160 @@
+"""ctypes binding of the C ABI declared in include/xdit_amd_attn.h.
+
+The shared library is built in-tree by `xdit_amd.build` (hipcc, gfx950).  Loading never
+falls back to anything else: if the library is missing, `lib()` raises.
+"""
+import ctypes
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libxdit_amd_attn.so")
+ABI_VERSION = 1
+
+XDIT_OK = 0
+XDIT_ERR_INVALID_ARG = -1
+XDIT_ERR_UNSUPPORTED = -2
+XDIT_ERR_LAUNCH = -3
+
+DTYPE_BF16, DTYPE_FP16, DTYPE_FP32, DTYPE_FP8_E4M3FN = 0, 1, 2, 3
+
+
+class Strides(ctypes.Structure):
+    _fields_ = [("b", ctypes.c_int64), ("h", ctypes.c_int64), ("s", ctypes.c_int64)]
+
+
+class AttnArgs(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32),
+        ("out_dtype", ctypes.c_int32),
+        ("causal", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
+        ("Sq", ctypes.c_int64),
+        ("Sk", ctypes.c_int64),
+        ("Sk2", ctypes.c_int64),
+        ("softmax_scale", ctypes.c_float),
+        ("reserved1", ctypes.c_float),
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("k2", ctypes.c_void_p),
+        ("v2", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("q_stride", Strides),
+        ("k_stride", Strides),
+        ("v_stride", Strides),
+        ("k2_stride", Strides),
+        ("v2_stride", Strides),
+        ("out_stride", Strides),
+        ("lse_stride_b", ctypes.c_int64),
+        ("lse_stride_h", ctypes.c_int64),
+        ("q_descale", ctypes.c_void_p),
+        ("k_descale", ctypes.c_void_p),
+        ("v_descale", ctypes.c_void_p),
+        ("descale_stride_b", ctypes.c_int64),
+        ("descale_stride_h", ctypes.c_int64),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+class MergeArgs(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("block_dtype", ctypes.c_int32),
+        ("final_dtype", ctypes.c_int32),
+        ("first", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
+        ("S", ctypes.c_int64),
+        ("acc_out", ctypes.c_void_p),
+        ("acc_lse", ctypes.c_void_p),
+        ("block_out", ctypes.c_void_p),
+        ("block_lse", ctypes.c_void_p),
+        ("final_out", ctypes.c_void_p),
+        ("acc_out_stride", Strides),
+        ("block_out_stride", Strides),
+        ("final_out_stride", Strides),
+        ("acc_lse_stride", Strides),
+        ("block_lse_stride", Strides),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+class QuantArgs(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("in_dtype", ctypes.c_int32),
+        ("per_tensor", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("S", ctypes.c_int64),
+        ("x", ctypes.c_void_p),
+        ("y", ctypes.c_void_p),
+        ("descale", ctypes.c_void_p),
+        ("x_stride", Strides),
+        ("y_stride", Strides),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+EXPORTS = ("xdit_attn_fwd", "xdit_lse_merge", "xdit_fp8_quant", "xdit_attn_last_error", "xdit_attn_abi_version")
+
+_lib = None
+_lock = threading.Lock()
+
+
+def lib():
+    """Return the loaded shared library (loading it on first use)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -m xdit_amd.build` (hipcc, gfx950). "
+                "There is no fallback path." % LIB_PATH
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        L.xdit_attn_fwd.argtypes = [ctypes.POINTER(AttnArgs)]
+        L.xdit_attn_fwd.restype = ctypes.c_int
+        L.xdit_lse_merge.argtypes = [ctypes.POINTER(MergeArgs)]
+        L.xdit_lse_merge.restype = ctypes.c_int
+        L.xdit_fp8_quant.argtypes = [ctypes.POINTER(QuantArgs)]
+        L.xdit_fp8_quant.restype = ctypes.c_int
+        L.xdit_attn_last_error.argtypes = []
+        L.xdit_attn_last_error.restype = ctypes.c_char_p
+        L.xdit_attn_abi_version.argtypes = []
+        L.xdit_attn_abi_version.restype = ctypes.c_int
+        v = L.xdit_attn_abi_version()
+        if v != ABI_VERSION:
+            raise RuntimeError("ABI version %d of %s != binding version %d" % (v, LIB_PATH, ABI_VERSION))
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().xdit_attn_last_error().decode("utf-8", "replace")
+
+
+def check(rc):
+    """Map a C status to the Python exception the reference's style uses:
+    ValueError for argument errors, NotImplementedError for unsupported options,
+    RuntimeError for launch failures."""
+    if rc == XDIT_OK:
+        return
+    msg = last_error()
+    if rc == XDIT_ERR_INVALID_ARG:
+        raise ValueError(msg)
+    if rc == XDIT_ERR_UNSUPPORTED:
+        raise NotImplementedError(msg)
+    raise RuntimeError(msg)

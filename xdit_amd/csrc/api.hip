@@ -1,0 +1,177 @@
+// C ABI of the attention hot path: argument validation, kernel selection, launch.
+// Nothing here allocates device memory or synchronises; every launch goes to the caller's stream.
+#include "../../include/xdit_amd_attn.h"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "common.h"
+#include "launchers.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int elem_size(int dtype) {
+  switch (dtype) {
+    case XDIT_DTYPE_BF16:
+    case XDIT_DTYPE_FP16: return 2;
+    case XDIT_DTYPE_FP32: return 4;
+    case XDIT_DTYPE_FP8_E4M3FN: return 1;
+    default: return 0;
+  }
+}
+
+// Every row of a tensor must start on a 16-byte boundary: base aligned, strides multiples of
+// 16 bytes.  The S stride must also keep 64 rows within a 32-bit byte offset (tile loads use
+// "64-bit uniform base + 32-bit per-lane offset" addressing).
+int check_tensor(const char* name, const void* p, const xdit_strides& st, int esize, int D) {
+  if (p == nullptr) return fail(XDIT_ERR_INVALID_ARG, "%s is NULL", name);
+  if (!aligned16(p)) return fail(XDIT_ERR_INVALID_ARG, "%s is not 16-byte aligned", name);
+  const int64_t m = 16 / esize;
+  if (st.b % m || st.h % m || st.s % m)
+    return fail(XDIT_ERR_INVALID_ARG, "%s: strides (%lld,%lld,%lld) must be multiples of %lld elements",
+                name, (long long)st.b, (long long)st.h, (long long)st.s, (long long)m);
+  if (st.s < D) return fail(XDIT_ERR_INVALID_ARG, "%s: S stride %lld is smaller than head_dim %d", name, (long long)st.s, D);
+  if (st.b < 0 || st.h < 0) return fail(XDIT_ERR_INVALID_ARG, "%s: negative stride", name);
+  if (st.s * esize >= (int64_t(1) << 25))
+    return fail(XDIT_ERR_INVALID_ARG, "%s: S stride of %lld bytes is too large", name, (long long)(st.s * esize));
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* xdit_attn_last_error(void) { return g_err; }
+
+int xdit_attn_abi_version(void) { return XDIT_ATTN_ABI_VERSION; }
+
+int xdit_attn_fwd(const xdit_attn_args* a) {
+  g_err[0] = 0;
+  if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
+  if (a->struct_size != sizeof(xdit_attn_args))
+    return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_attn_args));
+  const int es = elem_size(a->dtype);
+  if (es == 0) return fail(XDIT_ERR_INVALID_ARG, "unknown dtype %d", a->dtype);
+  if (a->causal != 0) return fail(XDIT_ERR_UNSUPPORTED, "causal attention is not implemented (DiT attention is non-causal)");
+  if (a->B <= 0 || a->H <= 0) return fail(XDIT_ERR_INVALID_ARG, "B=%d H=%d must be positive", a->B, a->H);
+  if (a->Sq <= 0 || a->Sk <= 0 || a->Sk2 < 0)
+    return fail(XDIT_ERR_INVALID_ARG, "Sq=%lld Sk=%lld Sk2=%lld: need Sq>0, Sk>0, Sk2>=0", (long long)a->Sq, (long long)a->Sk, (long long)a->Sk2);
+  if (a->Sq > (int64_t(1) << 30) || a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30))
+    return fail(XDIT_ERR_INVALID_ARG, "sequence length above 2^30");
+  if ((int64_t)a->B * a->H * ((a->Sq + 31) / 32) > (int64_t(1) << 30))
+    return fail(XDIT_ERR_INVALID_ARG, "B*H*Sq too large for one launch");
+  if (!(a->softmax_scale > 0.f) || !std::isfinite(a->softmax_scale))
+    return fail(XDIT_ERR_INVALID_ARG, "softmax_scale must be finite and > 0");
+  if (a->D <= 0 || a->D % 8 != 0 || a->D > 256) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d: need a multiple of 8, at most 256", a->D);
+
+  int out_dtype = a->out_dtype;
+  if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
+    if (out_dtype != XDIT_DTYPE_BF16 && out_dtype != XDIT_DTYPE_FP16)
+      return fail(XDIT_ERR_INVALID_ARG, "fp8 inputs need a bf16 or fp16 output");
+  } else if (out_dtype != a->dtype) {
+    return fail(XDIT_ERR_INVALID_ARG, "out_dtype %d must equal dtype %d", out_dtype, a->dtype);
+  }
+  int rc;
+  if ((rc = check_tensor("q", a->q, a->q_stride, es, a->D))) return rc;
+  if ((rc = check_tensor("k", a->k, a->k_stride, es, a->D))) return rc;
+  if ((rc = check_tensor("v", a->v, a->v_stride, es, a->D))) return rc;
+  if (a->Sk2 > 0) {
+    if ((rc = check_tensor("k2", a->k2, a->k2_stride, es, a->D))) return rc;
+    if ((rc = check_tensor("v2", a->v2, a->v2_stride, es, a->D))) return rc;
+  }
+  if ((rc = check_tensor("out", a->out, a->out_stride, elem_size(out_dtype), a->D))) return rc;
+  if (a->lse != nullptr && (a->lse_stride_b < 0 || a->lse_stride_h < a->Sq))
+    return fail(XDIT_ERR_INVALID_ARG, "lse strides (%lld,%lld) do not hold Sq=%lld rows", (long long)a->lse_stride_b, (long long)a->lse_stride_h, (long long)a->Sq);
+
+  xdit::AttnParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.q = a->q; p.k = a->k; p.v = a->v; p.k2 = a->k2; p.v2 = a->v2; p.out = a->out; p.lse = a->lse;
+  p.qs_b = a->q_stride.b; p.qs_h = a->q_stride.h; p.qs_s = a->q_stride.s;
+  p.ks_b = a->k_stride.b; p.ks_h = a->k_stride.h; p.ks_s = a->k_stride.s;
+  p.vs_b = a->v_stride.b; p.vs_h = a->v_stride.h; p.vs_s = a->v_stride.s;
+  p.k2s_b = a->k2_stride.b; p.k2s_h = a->k2_stride.h; p.k2s_s = a->k2_stride.s;
+  p.v2s_b = a->v2_stride.b; p.v2s_h = a->v2_stride.h; p.v2s_s = a->v2_stride.s;
+  p.os_b = a->out_stride.b; p.os_h = a->out_stride.h; p.os_s = a->out_stride.s;
+  p.ls_b = a->lse_stride_b; p.ls_h = a->lse_stride_h;
+  p.q_descale = a->q_descale; p.k_descale = a->k_descale; p.v_descale = a->v_descale;
+  p.ds_b = a->descale_stride_b; p.ds_h = a->descale_stride_h;
+  p.B = a->B; p.H = a->H;
+  p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
+  p.scale = a->softmax_scale;
+  hipStream_t stream = (hipStream_t)a->stream;
+
+  hipError_t e;
+  if ((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64)) {
+    e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, a->D, stream);
+  } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
+    if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
+    e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, stream);
+  } else {
+    if (a->D > 128) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d above 128 is not implemented", a->D);
+    e = xdit::launch_attn_fwd_f32(p, a->dtype, a->D, stream);
+  }
+  if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
+  return XDIT_OK;
+}
+
+int xdit_lse_merge(const xdit_merge_args* a) {
+  g_err[0] = 0;
+  if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
+  if (a->struct_size != sizeof(xdit_merge_args))
+    return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_merge_args));
+  if (a->block_dtype != XDIT_DTYPE_BF16 && a->block_dtype != XDIT_DTYPE_FP16 && a->block_dtype != XDIT_DTYPE_FP32)
+    return fail(XDIT_ERR_INVALID_ARG, "block_dtype %d must be bf16, fp16 or fp32", a->block_dtype);
+  if (a->B <= 0 || a->H <= 0 || a->S <= 0) return fail(XDIT_ERR_INVALID_ARG, "B, H, S must be positive");
+  if (a->D <= 0 || a->D % 8 != 0) return fail(XDIT_ERR_INVALID_ARG, "head_dim %d must be a positive multiple of 8", a->D);
+  if (a->S > (int64_t(1) << 30)) return fail(XDIT_ERR_INVALID_ARG, "S above 2^30");
+  if (a->acc_lse == nullptr || a->block_lse == nullptr) return fail(XDIT_ERR_INVALID_ARG, "acc_lse / block_lse is NULL");
+  int rc;
+  xdit_strides big = a->acc_out_stride;
+  if ((rc = check_tensor("acc_out", a->acc_out, big, 4, a->D))) return rc;
+  if ((rc = check_tensor("block_out", a->block_out, a->block_out_stride, elem_size(a->block_dtype), a->D))) return rc;
+  if (a->final_out != nullptr) {
+    if (a->final_dtype != XDIT_DTYPE_BF16 && a->final_dtype != XDIT_DTYPE_FP16 && a->final_dtype != XDIT_DTYPE_FP32)
+      return fail(XDIT_ERR_INVALID_ARG, "final_dtype %d must be bf16, fp16 or fp32", a->final_dtype);
+    if ((rc = check_tensor("final_out", a->final_out, a->final_out_stride, elem_size(a->final_dtype), a->D))) return rc;
+  }
+  xdit::MergeParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.acc_out = a->acc_out; p.acc_lse = a->acc_lse; p.block_out = a->block_out; p.block_lse = a->block_lse;
+  p.final_out = a->final_out;
+  p.ao_b = a->acc_out_stride.b; p.ao_h = a->acc_out_stride.h; p.ao_s = a->acc_out_stride.s;
+  p.bo_b = a->block_out_stride.b; p.bo_h = a->block_out_stride.h; p.bo_s = a->block_out_stride.s;
+  p.fo_b = a->final_out_stride.b; p.fo_h = a->final_out_stride.h; p.fo_s = a->final_out_stride.s;
+  p.al_b = a->acc_lse_stride.b; p.al_h = a->acc_lse_stride.h; p.al_s = a->acc_lse_stride.s;
+  p.bl_b = a->block_lse_stride.b; p.bl_h = a->block_lse_stride.h; p.bl_s = a->block_lse_stride.s;
+  p.B = a->B; p.H = a->H; p.S = (int)a->S; p.D = a->D;
+  p.first = a->first;
+  p.rows = (int64_t)a->B * a->H * a->S;
+  if (p.rows * (a->D / 8) > (int64_t(1) << 38)) return fail(XDIT_ERR_INVALID_ARG, "tensor too large for one launch");
+  hipError_t e = xdit::launch_lse_merge(p, a->block_dtype, a->final_dtype, (hipStream_t)a->stream);
+  if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "merge launch failed: %s", hipGetErrorString(e));
+  return XDIT_OK;
+}
+
+int xdit_fp8_quant(const xdit_quant_args* a) {
+  g_err[0] = 0;
+  if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
+  if (a->struct_size != sizeof(xdit_quant_args))
+    return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_quant_args));
+  return fail(XDIT_ERR_UNSUPPORTED, "fp8 quantiser is not implemented yet");
+}
+
+}  // extern "C"

@@ -1,0 +1,354 @@
+// Non-causal attention forward for 16-bit inputs (bf16 / fp16) on gfx950, head_dim 64 or 128.
+//
+// Work decomposition
+//   workgroup = 256 threads = 4 wavefronts; it owns 128 query rows of one (batch, head);
+//   wavefront w owns rows [32w, 32w+32).  Keys/values stream through LDS in tiles of 64 keys,
+//   double buffered, filled by direct global->LDS loads (16 bytes per lane).
+//
+// MFMA orientation (v_mfma_f32_32x32x16_{bf16,f16}; A is 32x16, B is 16x32, lane l holds row/col
+// l%32 and the 8 contraction elements 8*(l/32)..+7; the 32x32 result puts column l%32 and rows
+// 8*(i/4) + 4*(l/32) + i%4, i = 0..15, in lane l):
+//   S^T = K Q^T    A = K tile rows (keys), B = Q^T (kept in registers for the whole kernel)
+//   O^T = V^T P^T  A = V^T (read transposed from LDS with ds_read_b64_tr_b16), B = P^T
+// Computing the transposed products makes every lane own ONE query (column l%32): the softmax
+// row statistics are per-lane scalars (one exchange between the two wavefront halves per tile),
+// and the S^T accumulator registers are, after conversion to 16 bit, exactly the B operand of
+// the second product, so P never goes through LDS.
+//
+// LDS layout: a K (or V) tile is 64 rows of D 16-bit elements.  K is read with ds_read_b128
+// (lane -> one key row, 16 bytes), V with ds_read_b64_tr_b16 (16-lane group -> 4 key rows x 32
+// bytes).  A direct global->LDS load writes lane i at LDS offset base + 16*i, i.e. one 1 KiB
+// contiguous piece per wavefront instruction, so padding can only go BETWEEN those pieces.  Each
+// piece therefore holds rows {g, g+NG, g+2NG, ...} (NG pieces per tile) and pieces are
+// 1024 + PAD bytes apart: rows that are read together (consecutive rows) then sit in different
+// pieces, PAD bytes apart in bank space (PAD = 16 for the 16-byte K reads, 64 for the 64-byte V
+// reads), which makes both read patterns bank-conflict free while every read address is one
+// per-lane base plus a compile-time immediate.
+#include "common.h"
+#include "launchers.h"
+
+namespace xdit {
+
+constexpr int kRowsPerWave = 32;
+constexpr int kWaves = 4;
+constexpr int kRowsPerBlock = kRowsPerWave * kWaves;  // 128 query rows per workgroup
+constexpr int kKeysPerTile = 64;
+// A row maximum is replaced only when it grows by more than this many powers of two, so the
+// rescale of the output accumulator is skipped on almost every tile; exponentials stay <= 2^8.
+constexpr float kLazyRescaleLog2 = 8.0f;
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<__bf16> {
+  typedef bf16x8 vec8;
+  typedef bf16x2 vec2;
+  static __device__ __forceinline__ f32x16 mma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<_Float16> {
+  typedef f16x8 vec8;
+  typedef f16x2 vec2;
+  static __device__ __forceinline__ f32x16 mma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// Tile geometry: ROWS_PER_PIECE rows fit one 1 KiB wavefront load, NG pieces per 64-key tile;
+// row r lives in piece r % NG at slot r / NG.
+template <int D> struct TileGeom {
+  static constexpr int ROW_BYTES = D * 2;
+  static constexpr int ROWS_PER_PIECE = 1024 / ROW_BYTES;
+  static constexpr int NG = kKeysPerTile / ROWS_PER_PIECE;
+  static constexpr int K_PITCH = 1024 + 16;
+  static constexpr int V_PITCH = 1024 + 64;
+  static constexpr int K_BYTES = NG * K_PITCH;
+  static constexpr int V_BYTES = NG * V_PITCH;
+  static constexpr int BUF_BYTES = K_BYTES + V_BYTES;
+};
+
+// Direct global->LDS load of 16 bytes per lane: lane i's data lands at LDS address lds + 16*i.
+// `base` (64-bit) and `lds` must be wavefront-uniform; `off` is the lane's byte offset from base.
+// Issued as inline assembly so that the compiler does not order later LDS reads of the OTHER
+// tile buffer behind it; completion is awaited explicitly with s_waitcnt vmcnt(0).
+__device__ __forceinline__ void load_lds_16(const void* base, unsigned off, unsigned lds) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds), "v"(off), "s"(base)
+      : "memory", "m0");
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void attn_fwd_16_kernel(const AttnParams p) {
+  typedef typename Mfma16<T>::vec8 vec8;
+  typedef typename Mfma16<T>::vec2 vec2;
+  typedef TileGeom<D> G;
+  constexpr int LOADS = G::NG / kWaves;  // 1 KiB pieces per wavefront per tile (K and V each)
+  constexpr int KSTEPS = D / 16;         // contraction steps of QK^T
+  constexpr int DBLOCKS = D / 32;        // 32-row blocks of O^T
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // 2 x [K tile | V tile]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  const int tile = xcd_tile_index(blockIdx.x, p.tiles_per_xcd);
+  if (tile >= p.total_tiles) return;
+  const int bh = tile / p.nq_tiles;
+  const int qt = tile - bh * p.nq_tiles;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+
+  // ---- Q fragments: B operand of S^T, lane = (query l32, contraction half hh) -------------
+  const int qrow = qt * kRowsPerBlock + wave * kRowsPerWave + l32;
+  const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
+  const T* qptr = (const T*)p.q + b * p.qs_b + h * p.qs_h + (int64_t)qrow_c * p.qs_s + hh * 8;
+  vec8 qf[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ks++) qf[ks] = *(const vec8*)(qptr + ks * 16);
+
+  // ---- direct global->LDS tile loads ------------------------------------------------------
+  // Piece g = 4i + wave (i < LOADS) of a tile holds rows g, g+NG, g+2NG, ...; within the
+  // wavefront load lane -> (slot = lane / lanes-per-row, 16-byte column = lane % lanes-per-row).
+  // A load is "uniform 64-bit tile base + per-lane 32-bit byte offset"; the offsets of a full
+  // tile of segment 1 never change and live in registers.
+  const T* kbase1 = (const T*)p.k + b * p.ks_b + h * p.ks_h;
+  const T* vbase1 = (const T*)p.v + b * p.vs_b + h * p.vs_h;
+  const T* kbase2 = p.Sk2 > 0 ? (const T*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
+  const T* vbase2 = p.Sk2 > 0 ? (const T*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
+  constexpr int LANES_PER_ROW = G::ROW_BYTES / 16;
+  const int ld_slot = lane / LANES_PER_ROW;
+  const unsigned ld_colb = (lane % LANES_PER_ROW) * 16;  // byte offset inside the row
+  unsigned koffs[LOADS], voffs[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; i++) {
+    const unsigned r = 4 * i + wave + G::NG * ld_slot;
+    koffs[i] = r * (unsigned)(p.ks_s * 2) + ld_colb;
+    voffs[i] = r * (unsigned)(p.vs_s * 2) + ld_colb;
+  }
+  const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS unsigned char*)smem;
+
+  const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
+  const int nt2 = (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  const int nt = nt1 + nt2;
+
+  auto issue_tile = [&](int t, int buf) {
+    const unsigned kdst = lds_base + buf * G::BUF_BYTES;
+    const unsigned vdst = kdst + G::K_BYTES;
+    if (t < nt1 && (t + 1) * kKeysPerTile <= p.Sk) {  // full tile of segment 1
+      const T* kb = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
+      const T* vb = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
+#pragma unroll
+      for (int i = 0; i < LOADS; i++) {
+        const int g = 4 * i + wave;
+        load_lds_16(kb, koffs[i], kdst + g * G::K_PITCH);
+        load_lds_16(vb, voffs[i], vdst + g * G::V_PITCH);
+      }
+    } else {  // partial tile and/or segment 2: recompute the offsets
+      const T* kb;
+      const T* vb;
+      unsigned kss, vss;
+      int valid;
+      if (t < nt1) {
+        kb = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
+        vb = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
+        kss = (unsigned)(p.ks_s * 2); vss = (unsigned)(p.vs_s * 2);
+        valid = p.Sk - t * kKeysPerTile;
+      } else {
+        kb = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
+        vb = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
+        kss = (unsigned)(p.k2s_s * 2); vss = (unsigned)(p.v2s_s * 2);
+        valid = p.Sk2 - (t - nt1) * kKeysPerTile;
+      }
+      const int last = (valid < kKeysPerTile ? valid : kKeysPerTile) - 1;
+#pragma unroll
+      for (int i = 0; i < LOADS; i++) {
+        const int g = 4 * i + wave;
+        int r = g + G::NG * ld_slot;
+        r = r < last ? r : last;  // rows past the end of the segment re-read its last row
+        load_lds_16(kb, (unsigned)r * kss + ld_colb, kdst + g * G::K_PITCH);
+        load_lds_16(vb, (unsigned)r * vss + ld_colb, vdst + g * G::V_PITCH);
+      }
+    }
+  };
+
+  // ---- LDS read addresses: one per-lane base each for K and V, the rest are immediates ------
+  // K fragment (A operand of S^T) for key block kb, step ks: row 32kb + l32, bytes 32ks + 16hh.
+  //   row -> piece (row % NG), slot (row / NG)
+  const int kbase_off = (l32 % G::NG) * G::K_PITCH + (l32 / G::NG) * G::ROW_BYTES + hh * 16;
+  constexpr int K_KB_STEP = (32 / G::NG) * G::ROW_BYTES;  // +32 rows = +32/NG slots
+  // V^T fragment (A operand of O^T) for d block db, key step j (16 keys), half rd (keys +0 / +8):
+  // as a SOURCE lane of the transposed read, lane (group g = lane/16, s = lane%16) supplies the
+  // 8 bytes at key row 16j + 8rd + 4hh + s/4, elements d = 32db + 16(g%2) + 4(s%4) .. +3; the
+  // read returns to lane (g, i) the four keys of that row group at d = 32db + 16(g%2) + i.
+  const int vsrc_row = 4 * hh + ((lane & 15) >> 2);  // row within the 16-key step, rd = 0
+  const int vbase_off = (vsrc_row % G::NG) * G::V_PITCH + (vsrc_row / G::NG) * G::ROW_BYTES +
+                        (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  // +8 rows (rd) and +16 rows (j): both keep row % NG pattern simple because NG is 8 or 16.
+  constexpr int V_RD_STEP = (G::NG == 16) ? 8 * G::V_PITCH : G::ROW_BYTES;  // NG=8: +8 rows = +1 slot
+  constexpr int V_J_STEP = (16 / G::NG) * G::ROW_BYTES;
+
+  // ---- online softmax state: one query per lane (both halves of the wavefront agree) ------
+  const float c = p.scale * kLog2e;  // logits are kept in log2 units
+  float m_used = -INFINITY;          // running (lazily updated) row maximum of the raw dot products
+  float l_part = 0.f;                // this lane's share of the running row sum
+  f32x16 oacc[DBLOCKS];
+#pragma unroll
+  for (int db = 0; db < DBLOCKS; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+
+  issue_tile(0, 0);
+  // Make the compiler account for the Q fragment loads here, before the loop: the tile loads
+  // above are invisible to its outstanding-load bookkeeping, so any wait it placed for a Q
+  // fragment inside the loop would also wait for the prefetch of the next tile.
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+v"(qf[ks]));
+
+  for (int t = 0; t < nt; t++) {
+    const int buf = t & 1;
+    // Tile t has landed (this thread's loads) and, after the barrier, everyone's; the barrier
+    // also means every wavefront is done reading the other buffer, which tile t+1 now overwrites.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (t + 1 < nt) issue_tile(t + 1, buf ^ 1);
+
+    const XDIT_LDS unsigned char* ktile =
+        (const XDIT_LDS unsigned char*)(smem + buf * G::BUF_BYTES) + kbase_off;
+    const XDIT_LDS unsigned char* vtile =
+        (const XDIT_LDS unsigned char*)(smem + buf * G::BUF_BYTES + G::K_BYTES) + vbase_off;
+
+    // ---- S^T = K Q^T : 2 blocks of 32 keys x 32 queries ---------------------------------
+    f32x16 sacc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        vec8 kf = *(const XDIT_LDS vec8*)(ktile + kb * K_KB_STEP + ks * 32);
+        sacc[kb] = Mfma16<T>::mma(kf, qf[ks], sacc[kb]);
+      }
+    }
+
+    // ---- mask keys past the end of the segment (only its last tile can be partial) -------
+    const int valid = (t < nt1) ? p.Sk - t * kKeysPerTile : p.Sk2 - (t - nt1) * kKeysPerTile;
+    if (valid < kKeysPerTile) {
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          int key = 32 * kb + 8 * (i >> 2) + 4 * hh + (i & 3);
+          if (key >= valid) sacc[kb][i] = -INFINITY;
+        }
+    }
+
+    // ---- online softmax ---------------------------------------------------------------
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[0][i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[1][i]);
+    mx = max_halves(mx);
+    const float m_new = fmaxf(m_used, mx);
+    const bool grow = (m_new - m_used) * c > kLazyRescaleLog2;  // true on the first tile (-inf)
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float alpha = fast_exp2((m_used - m_new) * c);  // 0 on the first tile
+      m_used = m_new;
+      l_part *= alpha;
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+    }
+    const float mc = m_used * c;
+    vec8 pf[4];  // P^T as B operands: pf[j] = keys 16j..16j+15 of this tile (permuted inside)
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        float p0 = fast_exp2(__builtin_fmaf(sacc[kb][i], c, -mc));
+        float p1 = fast_exp2(__builtin_fmaf(sacc[kb][i + 1], c, -mc));
+        l_part += p0 + p1;
+        f32x2 pp = {p0, p1};
+        vec2 pk = __builtin_convertvector(pp, vec2);
+        const int j = 2 * kb + (i >> 3);
+        pf[j][(i & 7)] = pk[0];
+        pf[j][(i & 7) + 1] = pk[1];
+      }
+    }
+
+    // ---- O^T += V^T P^T ------------------------------------------------------------------
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; db++) {
+        typedef __attribute__((ext_vector_type(8))) short s16x8;
+        s16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (XDIT_LDS s16x4*)(vtile + j * V_J_STEP + db * 64));
+        s16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (XDIT_LDS s16x4*)(vtile + j * V_J_STEP + db * 64 + V_RD_STEP));
+        s16x8 vv = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+        oacc[db] = Mfma16<T>::mma(__builtin_bit_cast(vec8, vv), pf[j], oacc[db]);
+      }
+    }
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------
+  const float l_tot = sum_halves(l_part);
+  const float inv = 1.0f / l_tot;
+  if (qrow < p.Sq) {
+    T* optr = (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; db++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        // registers 4a..4a+3 are d = 32db + 8a + 4hh + 0..3 of this lane's query
+        typedef __attribute__((ext_vector_type(4))) T vec4;
+        f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                   oacc[db][4 * a + 3] * inv};
+        vec4 ov = __builtin_convertvector(o, vec4);
+        *(vec4*)(optr + 32 * db + 8 * a + 4 * hh) = ov;
+      }
+    if (p.lse != nullptr && hh == 0) {
+      p.lse[b * p.ls_b + h * p.ls_h + qrow] = (m_used * c + fast_log2(l_tot)) * kLn2;
+    }
+  }
+}
+
+template <typename T, int D>
+static hipError_t launch_one(const AttnParams& q, dim3 grid, hipStream_t stream, bool& lds_ready) {
+  constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
+  if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    lds_ready = true;
+  }
+  hipLaunchKernelGGL((attn_fwd_16_kernel<T, D>), grid, dim3(256), lds, stream, q);
+  return hipGetLastError();
+}
+
+// Host-side launcher (called from the C ABI after argument validation).
+hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, hipStream_t stream) {
+  AttnParams q = p;
+  q.nq_tiles = (p.Sq + kRowsPerBlock - 1) / kRowsPerBlock;
+  q.total_tiles = p.B * p.H * q.nq_tiles;
+  q.tiles_per_xcd = (q.total_tiles + 7) / 8;
+  dim3 grid(q.tiles_per_xcd * 8);
+  static bool ready[4] = {false, false, false, false};
+  if (D == 128) {
+    return dtype_is_fp16 ? launch_one<_Float16, 128>(q, grid, stream, ready[0])
+                         : launch_one<__bf16, 128>(q, grid, stream, ready[1]);
+  } else if (D == 64) {
+    return dtype_is_fp16 ? launch_one<_Float16, 64>(q, grid, stream, ready[2])
+                         : launch_one<__bf16, 64>(q, grid, stream, ready[3]);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace xdit

@@ -1,0 +1,81 @@
+// Shared device-side types and helpers for the gfx950 attention kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace xdit {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+
+#define XDIT_LDS __attribute__((address_space(3)))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Parameters of one attention-forward launch (passed by value).
+struct AttnParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* k2;
+  const void* v2;
+  void* out;
+  float* lse;
+  int64_t qs_b, qs_h, qs_s;
+  int64_t ks_b, ks_h, ks_s;
+  int64_t vs_b, vs_h, vs_s;
+  int64_t k2s_b, k2s_h, k2s_s;
+  int64_t v2s_b, v2s_h, v2s_s;
+  int64_t os_b, os_h, os_s;
+  int64_t ls_b, ls_h;
+  const float* q_descale;
+  const float* k_descale;
+  const float* v_descale;
+  int64_t ds_b, ds_h;
+  int B, H;
+  int Sq, Sk, Sk2;
+  int nq_tiles;       // ceil(Sq / rows per workgroup)
+  int total_tiles;    // B * H * nq_tiles
+  int tiles_per_xcd;  // ceil(total_tiles / 8)
+  float scale;        // softmax scale
+};
+
+// Combine a value across the two 32-lane halves of a wavefront (lane l with lane l^32).
+// v_permlane32_swap(a, b) leaves {own a, other half's a} in the low half and
+// {other half's b, own b} in the high half, so with a == b both halves hold {own, other}.
+__device__ __forceinline__ float max_halves(float x) {
+  int xi = __builtin_bit_cast(int, x);
+  auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+  return fmaxf(__builtin_bit_cast(float, (int)r[0]), __builtin_bit_cast(float, (int)r[1]));
+}
+__device__ __forceinline__ float sum_halves(float x) {
+  int xi = __builtin_bit_cast(int, x);
+  auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+  return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// Workgroup index -> work tile, XCD-aware.  Workgroups are handed to the 8 XCDs round-robin
+// (workgroup i runs on XCD i % 8).  Giving XCD x the contiguous tile range
+// [x * tiles_per_xcd, (x+1) * tiles_per_xcd) keeps the query tiles of one (batch, head) — which
+// all stream the same K/V — on one XCD, so that K/V is fetched into that XCD's L2 once.
+__device__ __forceinline__ int xcd_tile_index(int block, int tiles_per_xcd) {
+  return (block & 7) * tiles_per_xcd + (block >> 3);
+}
+
+}  // namespace xdit

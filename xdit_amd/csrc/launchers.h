@@ -1,0 +1,33 @@
+// Host-side launch functions of the kernels, shared between the kernel files and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "common.h"
+
+namespace xdit {
+
+// Parameters of one merge launch (passed by value to the kernel).
+struct MergeParams {
+  float* acc_out;
+  float* acc_lse;
+  const void* block_out;
+  const float* block_lse;
+  void* final_out;
+  int64_t ao_b, ao_h, ao_s;
+  int64_t bo_b, bo_h, bo_s;
+  int64_t fo_b, fo_h, fo_s;
+  int64_t al_b, al_h, al_s;
+  int64_t bl_b, bl_h, bl_s;
+  int B, H, S, D;
+  int first;
+  int64_t rows;  // B * H * S
+};
+
+// dtype codes below are the C ABI's xdit_dtype values: 0 bf16, 1 fp16, 2 fp32, 3 fp8 e4m3fn.
+hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, hipStream_t stream);
+hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, hipStream_t stream);
+hipError_t launch_attn_fwd_f32(const AttnParams& p, int dtype, int D, hipStream_t stream);
+hipError_t launch_lse_merge(const MergeParams& p, int block_dtype, int final_dtype, hipStream_t stream);
+
+}  // namespace xdit

@@ -1,0 +1,131 @@
+// Fused ring online-softmax merge (one pass over HBM, fp32 arithmetic) for gfx950.
+//
+//   acc_out <- acc_out - sigmoid(block_lse - acc_lse) * (acc_out - block_out)
+//   acc_lse <- acc_lse - logsigmoid(acc_lse - block_lse)
+//
+// This is the formula torch's _SDPAMerger._merge_one uses
+// (torch/distributed/tensor/experimental/_context_parallel/_attention.py:181-182) and that
+// xDiT's legacy ring loop reaches through `update_out_and_lse`
+// (xfuser/core/long_ctx_attention/ring/ring_flash_attn.py:138).  `first` initialises the
+// accumulator from the block instead (the `out is None` branch of update_out_and_lse /
+// _attention.py:161-163), and `final_out`, when given, receives the merged rows in the block
+// dtype (the epilogue cast at ring_flash_attn.py:145) in the same pass.
+//
+// Memory-bound: every thread moves 8 consecutive head_dim elements (32 B of fp32 accumulator,
+// 16 B of 16-bit block) per row; a row's D/8 threads are adjacent lanes, so accumulator accesses
+// coalesce to full rows.  The lse values of a row are loaded by each of its threads (served by
+// one L1 line) and stored by the first.
+#include "common.h"
+#include "launchers.h"
+
+namespace xdit {
+
+template <typename T> struct Load8;
+template <> struct Load8<float> {
+  static __device__ __forceinline__ void ld(const void* p, float (&x)[8]) {
+    const f32x4* q = (const f32x4*)p;
+    f32x4 a = q[0], b = q[1];
+    for (int i = 0; i < 4; i++) { x[i] = a[i]; x[4 + i] = b[i]; }
+  }
+  static __device__ __forceinline__ void st(void* p, const float (&x)[8]) {
+    f32x4 a = {x[0], x[1], x[2], x[3]}, b = {x[4], x[5], x[6], x[7]};
+    ((f32x4*)p)[0] = a;
+    ((f32x4*)p)[1] = b;
+  }
+};
+template <> struct Load8<__bf16> {
+  static __device__ __forceinline__ void ld(const void* p, float (&x)[8]) {
+    bf16x8 v = *(const bf16x8*)p;
+    for (int i = 0; i < 8; i++) x[i] = (float)v[i];
+  }
+  static __device__ __forceinline__ void st(void* p, const float (&x)[8]) {
+    bf16x8 v;
+    for (int i = 0; i < 8; i++) v[i] = (__bf16)x[i];
+    *(bf16x8*)p = v;
+  }
+};
+template <> struct Load8<_Float16> {
+  static __device__ __forceinline__ void ld(const void* p, float (&x)[8]) {
+    f16x8 v = *(const f16x8*)p;
+    for (int i = 0; i < 8; i++) x[i] = (float)v[i];
+  }
+  static __device__ __forceinline__ void st(void* p, const float (&x)[8]) {
+    f16x8 v;
+    for (int i = 0; i < 8; i++) v[i] = (_Float16)x[i];
+    *(f16x8*)p = v;
+  }
+};
+
+// logsigmoid(x) = min(x, 0) - log1p(exp(-|x|)), the form torch evaluates.
+__device__ __forceinline__ float log_sigmoid(float x) {
+  return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
+}
+__device__ __forceinline__ float sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+template <typename TB, typename TF, bool HAS_FINAL>
+__global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p) {
+  const int tpr = p.D >> 3;  // threads per row
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = gid / tpr;
+  const int col = (int)(gid - row * tpr) * 8;
+  if (row >= p.rows) return;
+  // row -> (b, h, s); consecutive rows walk s fastest, then h, then b
+  const int s = (int)(row % p.S);
+  const int64_t bh = row / p.S;
+  const int h = (int)(bh % p.H);
+  const int b = (int)(bh / p.H);
+
+  const float* bl = p.block_lse + b * p.bl_b + h * p.bl_h + s * p.bl_s;
+  float* al = p.acc_lse + b * p.al_b + h * p.al_h + s * p.al_s;
+  float* ao = p.acc_out + b * p.ao_b + h * p.ao_h + s * p.ao_s + col;
+  const TB* bo = (const TB*)p.block_out + b * p.bo_b + h * p.bo_h + s * p.bo_s + col;
+
+  float xb[8], xo[8];
+  Load8<TB>::ld(bo, xb);
+  const float blse = *bl;
+  float new_lse;
+  if (p.first) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) xo[i] = xb[i];
+    new_lse = blse;
+  } else {
+    Load8<float>::ld(ao, xo);
+    const float lse = *al;
+    const float w = sigmoid(blse - lse);
+#pragma unroll
+    for (int i = 0; i < 8; i++) xo[i] = xo[i] - w * (xo[i] - xb[i]);
+    new_lse = lse - log_sigmoid(lse - blse);
+  }
+  Load8<float>::st(ao, xo);
+  if (col == 0) *al = new_lse;
+  if (HAS_FINAL) {
+    TF* fo = (TF*)p.final_out + b * p.fo_b + h * p.fo_h + s * p.fo_s + col;
+    Load8<TF>::st(fo, xo);
+  }
+}
+
+template <typename TB>
+static hipError_t launch_tb(const MergeParams& p, int final_dtype, hipStream_t stream) {
+  const int64_t threads = p.rows * (p.D >> 3);
+  dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+  if (p.final_out == nullptr) {
+    hipLaunchKernelGGL((lse_merge_kernel<TB, float, false>), grid, block, 0, stream, p);
+  } else if (final_dtype == 0) {
+    hipLaunchKernelGGL((lse_merge_kernel<TB, __bf16, true>), grid, block, 0, stream, p);
+  } else if (final_dtype == 1) {
+    hipLaunchKernelGGL((lse_merge_kernel<TB, _Float16, true>), grid, block, 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((lse_merge_kernel<TB, float, true>), grid, block, 0, stream, p);
+  }
+  return hipGetLastError();
+}
+
+// dtype codes: 0 bf16, 1 fp16, 2 fp32 (the C ABI's xdit_dtype values).
+hipError_t launch_lse_merge(const MergeParams& p, int block_dtype, int final_dtype, hipStream_t stream) {
+  if (block_dtype == 0) return launch_tb<__bf16>(p, final_dtype, stream);
+  if (block_dtype == 1) return launch_tb<_Float16>(p, final_dtype, stream);
+  if (block_dtype == 2) return launch_tb<float>(p, final_dtype, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace xdit

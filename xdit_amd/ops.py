@@ -1,0 +1,155 @@
+"""Tensor-level entry points: torch tensors in, C ABI calls out.
+
+Tensors are logical (B, H, S, D) with arbitrary B/H/S strides and a unit D stride, so both
+BHSD-contiguous tensors and BSHD-contiguous tensors viewed as BHSD are consumed without a copy.
+PyTorch is used for device memory and the current stream only.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {
+    torch.bfloat16: _lib.DTYPE_BF16,
+    torch.float16: _lib.DTYPE_FP16,
+    torch.float32: _lib.DTYPE_FP32,
+    torch.float8_e4m3fn: _lib.DTYPE_FP8_E4M3FN,
+}
+
+
+def _code(dtype):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise ValueError("unsupported dtype %s" % (dtype,))
+
+
+def _strides(t):
+    return _lib.Strides(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _check4(name, t, device):
+    if not isinstance(t, torch.Tensor) or t.ndim != 4:
+        raise ValueError("%s must be a 4-D tensor (B, H, S, D)" % name)
+    if t.device != device:
+        raise ValueError("%s is on %s, expected %s" % (name, t.device, device))
+    if not t.is_cuda:
+        raise RuntimeError("%s is not on a GPU: the attention kernels are HIP-only, there is no CPU path" % name)
+    if t.shape[-1] > 1 and t.stride(-1) != 1:
+        raise ValueError("%s must have a unit stride over head_dim" % name)
+
+
+def _stream(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
+             q_descale=None, k_descale=None, v_descale=None, out_dtype=None, out=None,
+             return_lse=True):
+    """Non-causal attention forward on logical BHSD tensors -> (out BHSD, lse (B,H,Sq) fp32).
+
+    `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
+    with `k`/`v`.  For fp8 (torch.float8_e4m3fn) inputs the descales are (B, H) fp32 tensors.
+    """
+    device = q.device
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check4(name, t, device)
+    if (k2 is None) != (v2 is None):
+        raise ValueError("k2 and v2 should be None or not None simultaneously.")
+    B, H, Sq, D = q.shape
+    if k.shape[0] != B or k.shape[1] != H or k.shape[3] != D or v.shape != k.shape:
+        raise ValueError("q %s, k %s, v %s do not agree (Hq must equal Hk)" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k, v must share a dtype")
+    Sk = k.shape[2]
+    Sk2 = 0
+    if k2 is not None:
+        _check4("k2", k2, device)
+        _check4("v2", v2, device)
+        if k2.shape[0] != B or k2.shape[1] != H or k2.shape[3] != D or v2.shape != k2.shape or k2.dtype != q.dtype or v2.dtype != q.dtype:
+            raise ValueError("joint k2/v2 do not match q/k/v")
+        Sk2 = k2.shape[2]
+    dt = _code(q.dtype)
+    if out_dtype is None:
+        out_dtype = torch.bfloat16 if q.dtype == torch.float8_e4m3fn else q.dtype
+    if softmax_scale is None:
+        softmax_scale = float(D) ** -0.5
+    if out is None:
+        out = torch.empty((B, H, Sq, D), dtype=out_dtype, device=device)
+    else:
+        _check4("out", out, device)
+        if tuple(out.shape) != (B, H, Sq, D) or out.dtype != out_dtype:
+            raise ValueError("out has the wrong shape or dtype")
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=device) if return_lse else None
+
+    a = _lib.AttnArgs()
+    a.struct_size = ctypes.sizeof(_lib.AttnArgs)
+    a.dtype = dt
+    a.out_dtype = _code(out_dtype)
+    a.causal = 1 if causal else 0
+    a.B, a.H, a.D = B, H, D
+    a.Sq, a.Sk, a.Sk2 = Sq, Sk, Sk2
+    a.softmax_scale = float(softmax_scale)
+    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    a.q_stride, a.k_stride, a.v_stride = _strides(q), _strides(k), _strides(v)
+    if k2 is not None and Sk2 > 0:
+        a.k2, a.v2 = k2.data_ptr(), v2.data_ptr()
+        a.k2_stride, a.v2_stride = _strides(k2), _strides(v2)
+    a.out = out.data_ptr()
+    a.out_stride = _strides(out)
+    if lse is not None:
+        a.lse = lse.data_ptr()
+        a.lse_stride_b, a.lse_stride_h = lse.stride(0), lse.stride(1)
+    keep = []
+    for name, d in (("q_descale", q_descale), ("k_descale", k_descale), ("v_descale", v_descale)):
+        if d is None:
+            continue
+        if q.dtype != torch.float8_e4m3fn:
+            raise ValueError("%s is only meaningful for fp8 inputs" % name)
+        if d.dtype != torch.float32 or tuple(d.shape) != (B, H) or d.device != device:
+            raise ValueError("%s must be a (B, H) fp32 tensor on %s" % (name, device))
+        d = d.contiguous()
+        keep.append(d)
+        setattr(a, name, d.data_ptr())
+        a.descale_stride_b, a.descale_stride_h = d.stride(0), d.stride(1)
+    a.stream = _stream(device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().xdit_attn_fwd(ctypes.byref(a)))
+    return out, lse
+
+
+def lse_merge(acc_out, acc_lse, block_out, block_lse, first=False, final_out=None):
+    """One fold of the ring merge, in place on (acc_out fp32 BHSD-logical, acc_lse fp32 BHS-logical).
+
+    All tensors are given as LOGICAL (B,H,S,D) / (B,H,S) views (any strides, unit D stride).
+    """
+    device = block_out.device
+    _check4("acc_out", acc_out, device)
+    _check4("block_out", block_out, device)
+    if acc_out.dtype != torch.float32 or acc_lse.dtype != torch.float32 or block_lse.dtype != torch.float32:
+        raise ValueError("acc_out, acc_lse and block_lse must be fp32")
+    B, H, S, D = block_out.shape
+    if tuple(acc_out.shape) != (B, H, S, D) or tuple(acc_lse.shape) != (B, H, S) or tuple(block_lse.shape) != (B, H, S):
+        raise ValueError("shape mismatch between accumulator and block")
+    a = _lib.MergeArgs()
+    a.struct_size = ctypes.sizeof(_lib.MergeArgs)
+    a.block_dtype = _code(block_out.dtype)
+    a.first = 1 if first else 0
+    a.B, a.H, a.D, a.S = B, H, D, S
+    a.acc_out, a.acc_lse = acc_out.data_ptr(), acc_lse.data_ptr()
+    a.block_out, a.block_lse = block_out.data_ptr(), block_lse.data_ptr()
+    a.acc_out_stride, a.block_out_stride = _strides(acc_out), _strides(block_out)
+    a.acc_lse_stride = _lib.Strides(acc_lse.stride(0), acc_lse.stride(1), acc_lse.stride(2))
+    a.block_lse_stride = _lib.Strides(block_lse.stride(0), block_lse.stride(1), block_lse.stride(2))
+    if final_out is not None:
+        _check4("final_out", final_out, device)
+        if tuple(final_out.shape) != (B, H, S, D):
+            raise ValueError("final_out shape mismatch")
+        a.final_out = final_out.data_ptr()
+        a.final_dtype = _code(final_out.dtype)
+        a.final_out_stride = _strides(final_out)
+    a.stream = _stream(device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().xdit_lse_merge(ctypes.byref(a)))
+    return acc_out, acc_lse
