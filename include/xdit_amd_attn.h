@@ -127,11 +127,14 @@ typedef struct {
 int xdit_lse_merge(const xdit_merge_args* args);
 
 /*
- * Per-(batch,head) abs-max fp8 quantiser: for every (b,h), scale = absmax(x[b,h]) / 448 (or the
- * value 1.0 if the slice is all zero), y = fp8_e4m3fn(x / scale), descale[b,h] = scale.
- * `per_tensor != 0` uses one abs-max over the whole tensor and broadcasts it to (B,H), which is
- * the reference's per_tensor_quant (attention_backend.py:606-615).
- * `workspace` must hold at least B*H floats... it is the descale output itself; no extra memory.
+ * Abs-max fp8 quantiser, the step in front of the fp8 forward:
+ *     scale = absmax(x) / 448 (1.0 if x is all zero) ;  y = fp8_e4m3fn(x / scale) ;  descale = scale
+ * `per_tensor != 0`: one abs-max over the whole tensor, broadcast to every (b,h) entry of
+ * `descale` — the reference's per_tensor_quant (attention_backend.py:606-615), whose descale is
+ * `scale.expand(B, H)`.  `per_tensor == 0`: one abs-max per (batch, head) slice.
+ * `scale_in != NULL` (device pointer to one float) supplies a static scale instead of the abs-max
+ * (the `scale=` argument of per_tensor_quant).  Values whose quotient exceeds 448 saturate.
+ * `descale` (B*H contiguous fp32) doubles as the reduction buffer; no other memory is used.
  */
 typedef struct {
   uint32_t struct_size;        /* = sizeof(xdit_quant_args) */
@@ -142,6 +145,7 @@ typedef struct {
   const void* x;               /* (B,H,S,D) in_dtype */
   void* y;                     /* (B,H,S,D) fp8 e4m3fn bytes */
   float* descale;              /* (B,H) fp32, contiguous */
+  const float* scale_in;       /* optional static scale, may be NULL */
   xdit_strides x_stride, y_stride;
   void* stream;
 } xdit_quant_args;

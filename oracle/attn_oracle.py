@@ -1,0 +1,243 @@
+"""CPU oracle for the attention hot path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, on the CPU in float64 (or float32 where noted), the arithmetic of the
+reference's single-device attention path.  Only `tests/`, `__graft_entry__.smoke()` and the
+`cpu_baseline` leg of `bench.py` may import it; the product (`xdit_amd/`) never does.
+
+What each function follows (paths relative to the xDiT source tree unless prefixed `torch:`,
+which is the PyTorch wheel the reference depends on):
+
+* `attn_fwd_ref`         softmax(Q K^T * scale) V and logsumexp, the contract of the registry
+                         adapters xfuser/core/distributed/attention_backend.py:504-516 (out, lse),
+                         :518-532 (math path, out only), :774-823 (AITER: scale = D**-0.5).
+* `merge_ref`            torch:distributed/tensor/experimental/_context_parallel/_attention.py:181-182
+                         (the sigmoid / logsigmoid form; yunchang's update_out_and_lse, reached at
+                         xfuser/core/long_ctx_attention/ring/ring_flash_attn.py:138, is the same).
+* `update_out_and_lse_ref`  first-call and layout semantics visible at ring_flash_attn.py:68-69,
+                         :138, :145-148 (BSHD accumulator, lse kept as (B,S,H,1)).
+* `ring_forward_ref`     the loop of ring_flash_attn.py:83-148 on one device (KV chunks visited
+                         in the order a rank would receive them), joint K/V on the first ("front")
+                         or last ("rear") step, :89-100.
+* `per_tensor_quant_ref` attention_backend.py:606-615.
+* `sdpa_cpu`             the body of `_sdpa_attn_call`, attention_backend.py:499-501 (used as the
+                         timed CPU baseline).
+
+Pinning (tests/test_oracle.py): brute force with math.fsum on tiny inputs; torch's own CPU
+ops `aten._scaled_dot_product_attention_math` and `aten._scaled_dot_product_flash_attention_for_cpu`;
+closed forms and invariants of the merge (log-add-exp identity, fold of any KV partition equals the
+single pass, -inf block is the identity, equal lse gives the mean); the C twin in attn_ref.c.
+The reference holds no golden vectors for this path, so values are pinned by those checks, and
+the tolerances (not values) come from the reference's tests.
+"""
+import math
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+
+# ----------------------------------------------------------------------------------------------
+# attention forward
+# ----------------------------------------------------------------------------------------------
+def attn_fwd_ref(q, k, v, softmax_scale=None, dtype=torch.float64, q_chunk=1024):
+    """(out, lse) for logical BHSD tensors, evaluated in `dtype` on the CPU.
+
+    out_i = sum_j softmax_j(scale * q_i.k_j) v_j ; lse_i = log sum_j exp(scale * q_i.k_j)
+    (natural log, scale included).  Query rows are processed in chunks to bound memory.
+    """
+    q = q.detach().to("cpu").to(dtype)
+    k = k.detach().to("cpu").to(dtype)
+    v = v.detach().to("cpu").to(dtype)
+    B, H, Sq, D = q.shape
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(D)
+    out = torch.empty((B, H, Sq, v.shape[-1]), dtype=dtype)
+    lse = torch.empty((B, H, Sq), dtype=dtype)
+    kt = k.transpose(-1, -2)
+    for s0 in range(0, Sq, q_chunk):
+        s = torch.matmul(q[:, :, s0:s0 + q_chunk], kt) * softmax_scale
+        m = s.max(dim=-1, keepdim=True).values
+        p = torch.exp(s - m)
+        l = p.sum(dim=-1, keepdim=True)
+        out[:, :, s0:s0 + q_chunk] = torch.matmul(p, v) / l
+        lse[:, :, s0:s0 + q_chunk] = (m + torch.log(l)).squeeze(-1)
+    return out, lse
+
+
+def attn_rows_ref(q, k, v, rows, softmax_scale=None, dtype=torch.float64):
+    """(out, lse) for the given query rows only (all batches and heads, full K/V).
+    Used to probe long sequences where the full reference is too expensive."""
+    idx = torch.as_tensor(rows, dtype=torch.long)
+    return attn_fwd_ref(q.detach().to("cpu")[:, :, idx], k, v, softmax_scale, dtype)
+
+
+def attn_bruteforce(q, k, v, softmax_scale):
+    """Pure-Python restatement with exactly rounded sums (math.fsum) for tiny inputs.
+    q: [Sq][D], k: [Sk][D], v: [Sk][Dv] nested lists of floats -> (out [Sq][Dv], lse [Sq])."""
+    out, lse = [], []
+    for qi in q:
+        s = [softmax_scale * math.fsum(a * b for a, b in zip(qi, kj)) for kj in k]
+        m = max(s)
+        e = [math.exp(x - m) for x in s]
+        l = math.fsum(e)
+        lse.append(m + math.log(l))
+        out.append([math.fsum(e[j] * v[j][d] for j in range(len(k))) / l for d in range(len(v[0]))])
+    return out, lse
+
+
+def sdpa_cpu(q, k, v):
+    """What the reference's default SDPA adapter runs (attention_backend.py:499-501), on CPU."""
+    return F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False)
+
+
+# ----------------------------------------------------------------------------------------------
+# ring merge
+# ----------------------------------------------------------------------------------------------
+def merge_ref(out, lse, block_out, block_lse, dtype=torch.float64):
+    """One fold.  out/block_out: (..., D); lse/block_lse: (...) (no trailing 1).
+    out' = out - sigmoid(block_lse - lse) * (out - block_out)
+    lse' = lse - logsigmoid(lse - block_lse)"""
+    out = out.to(dtype)
+    block_out = block_out.to(dtype)
+    lse = lse.to(dtype).unsqueeze(-1)
+    block_lse = block_lse.to(dtype).unsqueeze(-1)
+    new_out = out - torch.sigmoid(block_lse - lse) * (out - block_out)
+    new_lse = lse - F.logsigmoid(lse - block_lse)
+    return new_out, new_lse.squeeze(-1)
+
+
+def merge_closed_form(out, lse, block_out, block_lse):
+    """The same fold written as the log-add-exp identity (float64):
+    L = log(e^l1 + e^l2), o = (e^l1 o1 + e^l2 o2) / e^L."""
+    l1 = lse.double().unsqueeze(-1)
+    l2 = block_lse.double().unsqueeze(-1)
+    L = torch.logaddexp(l1, l2)
+    o = torch.exp(l1 - L) * out.double() + torch.exp(l2 - L) * block_out.double()
+    return o, L.squeeze(-1)
+
+
+def update_out_and_lse_ref(out, lse, block_out, block_lse, dtype=torch.float32):
+    """The legacy ring's accumulator update in its own layout: block_out (B,S,H,D),
+    block_lse (B,H,S); accumulator out fp32 (B,S,H,D), lse fp32 (B,S,H,1).
+    First call (out is None) initialises from the block."""
+    if out is None:
+        return block_out.to(dtype), block_lse.to(dtype).transpose(-2, -1).unsqueeze(-1)
+    bl = block_lse.to(dtype).transpose(-2, -1).unsqueeze(-1)
+    bo = block_out.to(dtype)
+    new_out = out - torch.sigmoid(bl - lse) * (out - bo)
+    new_lse = lse - F.logsigmoid(lse - bl)
+    return new_out, new_lse
+
+
+def ring_forward_ref(q, k, v, n_chunks, order=None, softmax_scale=None, joint_k=None, joint_v=None,
+                     joint_strategy="none", chunk_dtype=None, dtype=torch.float64):
+    """Single-device restatement of the ring loop on BHSD tensors: K/V are split into `n_chunks`
+    contiguous chunks visited in `order` (default: the order rank 0 sees, [0, P-1, ..., 1]); each
+    step's (out_i, lse_i) is folded with `merge_ref`.  `chunk_dtype` optionally rounds each
+    per-chunk output (as a bf16 kernel would) before the fold."""
+    P = n_chunks
+    if order is None:
+        order = [0] + list(range(P - 1, 0, -1))
+    ks = k.chunk(P, dim=2)
+    vs = v.chunk(P, dim=2)
+    out = lse = None
+    for step, c in enumerate(order):
+        kk, vv = ks[c], vs[c]
+        if joint_strategy == "front" and step == 0:
+            kk, vv = torch.cat([joint_k, kk], 2), torch.cat([joint_v, vv], 2)
+        elif joint_strategy == "rear" and step == P - 1:
+            kk, vv = torch.cat([kk, joint_k], 2), torch.cat([vv, joint_v], 2)
+        bo, bl = attn_fwd_ref(q, kk, vv, softmax_scale, dtype)
+        if chunk_dtype is not None:
+            bo = bo.to(chunk_dtype).to(dtype)
+            bl = bl.float().to(dtype)
+        if out is None:
+            out, lse = bo, bl
+        else:
+            out, lse = merge_ref(out, lse, bo, bl, dtype)
+    return out, lse
+
+
+# ----------------------------------------------------------------------------------------------
+# fp8
+# ----------------------------------------------------------------------------------------------
+FP8_MAX = 448.0  # torch.finfo(torch.float8_e4m3fn).max
+
+
+def per_tensor_quant_ref(x, scale=None):
+    """attention_backend.py:606-615: scale = absmax(x)/448 over the WHOLE tensor, y = fp8(x/scale),
+    descale broadcast to x.shape[:2]."""
+    x = x.to(torch.float32)
+    if scale is None:
+        scale = torch.abs(x).max() / FP8_MAX
+    y = x / scale
+    return y.to(torch.float8_e4m3fn), scale.expand(*x.shape[:2]).to(torch.float32)
+
+
+def per_head_quant_ref(x):
+    """Per-(batch, head) abs-max quantiser for a BHSD tensor: scale[b,h] = absmax(x[b,h])/448
+    (1.0 for an all-zero slice)."""
+    x = x.to(torch.float32)
+    amax = x.abs().amax(dim=(2, 3))
+    scale = torch.where(amax > 0, amax / FP8_MAX, torch.ones_like(amax))
+    y = (x / scale[:, :, None, None]).to(torch.float8_e4m3fn)
+    return y, scale
+
+
+def dequant(y, scale):
+    """fp8 bytes + (B,H) scales -> float32 BHSD."""
+    return y.to(torch.float32) * scale[:, :, None, None].to(torch.float32)
+
+
+# ----------------------------------------------------------------------------------------------
+# seeded inputs of the benchmark configurations (generated on the CPU in fp32)
+# ----------------------------------------------------------------------------------------------
+def _randn(shape, gen):
+    return torch.randn(shape, generator=gen, dtype=torch.float32)
+
+
+def _rmsnorm_heads(x, gain, eps=1e-6):
+    """Per-head RMSNorm over head_dim with one gain vector of size head_dim
+    (the shape of attn.norm_q / norm_k, transformer_flux.py:120-121)."""
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * gain
+
+
+def make_qkv(B, H, S, D, seed, rmsnorm=False, dtype=torch.float32):
+    """q, k, v ~ N(0,1) in BHSD from `seed`; with `rmsnorm`, q and k get a per-head RMSNorm with
+    gains ~ U(0.8, 1.2)."""
+    g = torch.Generator().manual_seed(seed)
+    q = _randn((B, H, S, D), g)
+    k = _randn((B, H, S, D), g)
+    v = _randn((B, H, S, D), g)
+    if rmsnorm:
+        gq = 0.8 + 0.4 * torch.rand(D, generator=g)
+        gk = 0.8 + 0.4 * torch.rand(D, generator=g)
+        q = _rmsnorm_heads(q, gq)
+        k = _rmsnorm_heads(k, gk)
+    return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+CONFIGS = {
+    # name: (B, H, S, D, seed, rmsnorm, dtype)
+    "c1_pixart512": (1, 16, 1024, 72, 1001, False, torch.float32),
+    "c2_flux1024": (1, 24, 4608, 128, 1002, True, torch.bfloat16),
+    "c4_hunyuan720p_shard": (1, 3, 118800 + 256, 128, 1004, True, torch.bfloat16),
+    "c5_wan720p_shard_fp8": (1, 5, 75600, 128, 1005, False, torch.float8_e4m3fn),
+}
+
+
+def make_config(name, S=None):
+    """Inputs of a named configuration (optionally with a shorter sequence for CPU-sized tests).
+    Returns a dict with q, k, v (and q_descale, k_descale, v_descale for fp8)."""
+    B, H, S0, D, seed, rms, dtype = CONFIGS[name]
+    S = S0 if S is None else S
+    if dtype == torch.float8_e4m3fn:
+        q, k, v = make_qkv(B, H, S, D, seed, rms, torch.float32)
+        out = {}
+        for n, t in (("q", q), ("k", k), ("v", v)):
+            y, s = per_head_quant_ref(t)
+            out[n] = y
+            out[n + "_descale"] = s
+        return out
+    q, k, v = make_qkv(B, H, S, D, seed, rms, dtype)
+    return {"q": q, "k": k, "v": v}

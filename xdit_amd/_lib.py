@@ -99,6 +99,7 @@ class QuantArgs(ctypes.Structure):
         ("x", ctypes.c_void_p),
         ("y", ctypes.c_void_p),
         ("descale", ctypes.c_void_p),
+        ("scale_in", ctypes.c_void_p),
         ("x_stride", Strides),
         ("y_stride", Strides),
         ("stream", ctypes.c_void_p),

@@ -171,7 +171,30 @@ int xdit_fp8_quant(const xdit_quant_args* a) {
   if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
   if (a->struct_size != sizeof(xdit_quant_args))
     return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_quant_args));
-  return fail(XDIT_ERR_UNSUPPORTED, "fp8 quantiser is not implemented yet");
+  if (a->in_dtype != XDIT_DTYPE_BF16 && a->in_dtype != XDIT_DTYPE_FP16 && a->in_dtype != XDIT_DTYPE_FP32)
+    return fail(XDIT_ERR_INVALID_ARG, "in_dtype %d must be bf16, fp16 or fp32", a->in_dtype);
+  if (a->B <= 0 || a->H <= 0 || a->S <= 0) return fail(XDIT_ERR_INVALID_ARG, "B, H, S must be positive");
+  if (a->B * (int64_t)a->H > 65535) return fail(XDIT_ERR_INVALID_ARG, "B*H above 65535");
+  if (a->per_tensor && a->B * (int64_t)a->H > 1024) return fail(XDIT_ERR_INVALID_ARG, "per_tensor mode supports B*H <= 1024");
+  if (a->D <= 0 || a->D % 8 != 0) return fail(XDIT_ERR_INVALID_ARG, "head_dim %d must be a positive multiple of 8", a->D);
+  if (a->S > (int64_t(1) << 30)) return fail(XDIT_ERR_INVALID_ARG, "S above 2^30");
+  if (a->descale == nullptr) return fail(XDIT_ERR_INVALID_ARG, "descale is NULL");
+  int rc;
+  if ((rc = check_tensor("x", a->x, a->x_stride, elem_size(a->in_dtype), a->D))) return rc;
+  if (a->y == nullptr) return fail(XDIT_ERR_INVALID_ARG, "y is NULL");
+  if ((reinterpret_cast<uintptr_t>(a->y) & 7u) || a->y_stride.b % 8 || a->y_stride.h % 8 || a->y_stride.s % 8)
+    return fail(XDIT_ERR_INVALID_ARG, "y must be 8-byte aligned with strides that are multiples of 8");
+  if (a->y_stride.s < a->D) return fail(XDIT_ERR_INVALID_ARG, "y: S stride smaller than head_dim");
+  xdit::QuantParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.x = a->x; p.y = a->y; p.amax = a->descale; p.descale = a->descale; p.scale_in = a->scale_in;
+  p.xs_b = a->x_stride.b; p.xs_h = a->x_stride.h; p.xs_s = a->x_stride.s;
+  p.ys_b = a->y_stride.b; p.ys_h = a->y_stride.h; p.ys_s = a->y_stride.s;
+  p.B = a->B; p.H = a->H; p.S = (int)a->S; p.D = a->D;
+  p.per_tensor = a->per_tensor ? 1 : 0;
+  hipError_t e = xdit::launch_fp8_quant(p, a->in_dtype, (hipStream_t)a->stream);
+  if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "quantiser launch failed: %s", hipGetErrorString(e));
+  return XDIT_OK;
 }
 
 }  // extern "C"

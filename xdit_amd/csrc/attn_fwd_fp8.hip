@@ -1,5 +1,274 @@
+// Non-causal attention forward for fp8 (OCP e4m3fn) Q/K/V with per-(batch, head) fp32 descales,
+// head_dim 128, bf16 or fp16 output, fp32 log-sum-exp, on gfx950.
+//
+// Same structure as the 16-bit kernel (workgroup = 4 wavefronts x 32 query rows, 64-key K/V
+// tiles double buffered in LDS by direct global->LDS loads, transposed products so that each lane
+// owns one query), with v_mfma_f32_32x32x64_f8f6f4 for both products:
+//   S^T = K Q^T    A = K rows, B = Q^T (registers); contraction over head_dim, 64 per instruction.
+//                  A and B use the same lane->contraction-index map, so each lane simply holds the
+//                  32 contiguous bytes d = 64ks + 32(l/32) .. +31 of its row.
+//   O^T = V^T P^T  contraction over the 64 keys of the tile in ONE instruction per 32 rows of
+//                  head_dim.  P^T is the S^T accumulator converted to fp8 in register order, so
+//                  byte e = 16kb + i of lane (query, half hh) is key 32kb + 8(i/4) + 4hh + i%4;
+//                  V^T is fetched with ds_read_b64_tr_b8, whose source lanes are pointed at exactly
+//                  those key rows, so both operands agree on the byte -> key map.
+// P is scaled by 2^kPShift before the fp8 conversion so the bulk of the probabilities sits in
+// e4m3's normal range; the same factor is in the row sum, so it cancels in the output and is
+// subtracted from the log-sum-exp.  Logits are (q.k) * softmax_scale * q_descale * k_descale; the
+// output is multiplied by v_descale.
 #include "common.h"
 #include "launchers.h"
+
 namespace xdit {
-hipError_t launch_attn_fwd_fp8(const AttnParams&, int, hipStream_t) { return hipErrorNotSupported; }
+
+namespace fp8path {
+
+constexpr int kRowsPerWave = 32;
+constexpr int kWaves = 4;
+constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
+constexpr int kKeysPerTile = 64;
+constexpr int D = 128;
+constexpr float kPShift = 6.0f;           // P is scaled by 2^6 ...
+constexpr float kLazyRescaleLog2 = 2.0f;  // ... and the row max may lag by 2^2: P <= 2^8 < 448
+
+// LDS tile geometry: rows of 128 bytes, 8 rows per 1 KiB piece, 8 pieces per 64-key tile;
+// row r lives in piece r % 8 at slot r / 8.  Piece pitches pad by 16 B (K: 16-byte reads of 16
+// consecutive rows) and 32 B (V: 32-byte row segments of 8 rows) to spread the banks.
+constexpr int ROW_BYTES = 128;
+constexpr int NG = 8;
+constexpr int K_PITCH = 1024 + 16;
+constexpr int V_PITCH = 1024 + 32;
+constexpr int K_BYTES = NG * K_PITCH;
+constexpr int V_BYTES = NG * V_PITCH;
+constexpr int BUF_BYTES = K_BYTES + V_BYTES;
+constexpr int LOADS = NG / kWaves;  // 1 KiB pieces per wavefront per tile (K and V each)
+
+__device__ __forceinline__ void load_lds_16(const void* base, unsigned off, unsigned lds) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds), "v"(off), "s"(base)
+      : "memory", "m0");
 }
+
+template <typename TO>
+__global__ __launch_bounds__(256, 2) void attn_fwd_fp8_kernel(const AttnParams p) {
+  typedef unsigned char u8;
+  __shared__ __attribute__((aligned(1024))) u8 smem[2 * BUF_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  const int tile = xcd_tile_index(blockIdx.x, p.tiles_per_xcd);
+  if (tile >= p.total_tiles) return;
+  const int bh = tile / p.nq_tiles;
+  const int qt = tile - bh * p.nq_tiles;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+
+  // ---- Q fragments: 2 contraction steps x 32 bytes ---------------------------------------
+  const int qrow = qt * kRowsPerBlock + wave * kRowsPerWave + l32;
+  const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
+  const u8* qptr = (const u8*)p.q + b * p.qs_b + h * p.qs_h + (int64_t)qrow_c * p.qs_s + hh * 32;
+  i32x8 qf[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) {
+    i32x4 lo = *(const i32x4*)(qptr + ks * 64);
+    i32x4 hi = *(const i32x4*)(qptr + ks * 64 + 16);
+    qf[ks] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+
+  // ---- tile loads ------------------------------------------------------------------------
+  const u8* kbase1 = (const u8*)p.k + b * p.ks_b + h * p.ks_h;
+  const u8* vbase1 = (const u8*)p.v + b * p.vs_b + h * p.vs_h;
+  const u8* kbase2 = p.Sk2 > 0 ? (const u8*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
+  const u8* vbase2 = p.Sk2 > 0 ? (const u8*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
+  const int ld_slot = lane >> 3;                // 8 lanes per 128-byte row
+  const unsigned ld_colb = (lane & 7) * 16;
+  const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS u8*)smem;
+  const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
+  const int nt2 = (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  const int nt = nt1 + nt2;
+
+  auto issue_tile = [&](int t, int buf) {
+    const unsigned kdst = lds_base + buf * BUF_BYTES;
+    const unsigned vdst = kdst + K_BYTES;
+    const u8* kb;
+    const u8* vb;
+    unsigned kss, vss;
+    int valid;
+    if (t < nt1) {
+      kb = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
+      vb = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
+      kss = (unsigned)p.ks_s; vss = (unsigned)p.vs_s;
+      valid = p.Sk - t * kKeysPerTile;
+    } else {
+      kb = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
+      vb = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
+      kss = (unsigned)p.k2s_s; vss = (unsigned)p.v2s_s;
+      valid = p.Sk2 - (t - nt1) * kKeysPerTile;
+    }
+    const int last = (valid < kKeysPerTile ? valid : kKeysPerTile) - 1;
+#pragma unroll
+    for (int i = 0; i < LOADS; i++) {
+      const int g = 4 * i + wave;
+      int r = g + NG * ld_slot;
+      r = r < last ? r : last;  // rows past the end of the segment re-read its last row
+      load_lds_16(kb, (unsigned)r * kss + ld_colb, kdst + g * K_PITCH);
+      load_lds_16(vb, (unsigned)r * vss + ld_colb, vdst + g * V_PITCH);
+    }
+  };
+
+  // ---- LDS read bases ------------------------------------------------------------------------
+  // K fragment for key block kb, step ks: row 32kb + l32, bytes 64ks + 32hh .. +31.
+  const int kbase_off = (l32 & 7) * K_PITCH + (l32 >> 3) * ROW_BYTES + hh * 32;
+  // V^T fragment, read r (0..3), d block db: as a SOURCE lane of ds_read_b64_tr_b8, lane
+  // (group g = lane/16, s = lane%16) supplies 8 bytes of key row 16r + 8(s/8) + 4hh + (s/2)%4
+  // at d = 32db + 16(g%2) + 8(s%2); lane (g, i) receives d = 32db + 16(g%2) + i for the 8 keys
+  // 16r + 8(j/4) + 4hh + j%4, j = 0..7.
+  const int s16 = lane & 15;
+  const int vbase_off = (4 * hh + ((s16 >> 1) & 3)) * V_PITCH + (s16 >> 3) * ROW_BYTES +
+                        16 * ((lane >> 4) & 1) + 8 * (s16 & 1);
+
+  // ---- softmax state -------------------------------------------------------------------------
+  float sq = 1.f, sk = 1.f, sv = 1.f;
+  if (p.q_descale) sq = p.q_descale[b * p.ds_b + h * p.ds_h];
+  if (p.k_descale) sk = p.k_descale[b * p.ds_b + h * p.ds_h];
+  if (p.v_descale) sv = p.v_descale[b * p.ds_b + h * p.ds_h];
+  const float c = p.scale * sq * sk * kLog2e;
+  float m_used = -INFINITY;
+  float l_part = 0.f;
+  f32x16 oacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+
+  issue_tile(0, 0);
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) asm volatile("" : "+v"(qf[ks]));
+
+  for (int t = 0; t < nt; t++) {
+    const int buf = t & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (t + 1 < nt) issue_tile(t + 1, buf ^ 1);
+
+    const XDIT_LDS u8* ktile = (const XDIT_LDS u8*)(smem + buf * BUF_BYTES) + kbase_off;
+    const XDIT_LDS u8* vtile = (const XDIT_LDS u8*)(smem + buf * BUF_BYTES + K_BYTES) + vbase_off;
+
+    // ---- S^T = K Q^T ---------------------------------------------------------------------
+    f32x16 sacc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        i32x4 lo = *(const XDIT_LDS i32x4*)(ktile + kb * 4 * ROW_BYTES + ks * 64);
+        i32x4 hi = *(const XDIT_LDS i32x4*)(ktile + kb * 4 * ROW_BYTES + ks * 64 + 16);
+        i32x8 kf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[ks], sacc[kb], 0, 0, 0, 0, 0, 0);
+      }
+    }
+
+    const int valid = (t < nt1) ? p.Sk - t * kKeysPerTile : p.Sk2 - (t - nt1) * kKeysPerTile;
+    if (valid < kKeysPerTile) {
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          int key = 32 * kb + 8 * (i >> 2) + 4 * hh + (i & 3);
+          if (key >= valid) sacc[kb][i] = -INFINITY;
+        }
+    }
+
+    // ---- online softmax ---------------------------------------------------------------
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[0][i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[1][i]);
+    mx = max_halves(mx);
+    const float m_new = fmaxf(m_used, mx);
+    const bool grow = (m_new - m_used) * c > kLazyRescaleLog2;
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float alpha = fast_exp2((m_used - m_new) * c);
+      m_used = m_new;
+      l_part *= alpha;
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+    }
+    const float mc = m_used * c - kPShift;
+    i32x8 pf;  // P^T: byte 16kb + i
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+      for (int i = 0; i < 16; i += 4) {
+        float p0 = fast_exp2(__builtin_fmaf(sacc[kb][i], c, -mc));
+        float p1 = fast_exp2(__builtin_fmaf(sacc[kb][i + 1], c, -mc));
+        float p2 = fast_exp2(__builtin_fmaf(sacc[kb][i + 2], c, -mc));
+        float p3 = fast_exp2(__builtin_fmaf(sacc[kb][i + 3], c, -mc));
+        l_part += (p0 + p1) + (p2 + p3);
+        int w = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, w, true);
+        pf[4 * kb + (i >> 2)] = w;
+      }
+    }
+
+    // ---- O^T += V^T P^T ------------------------------------------------------------------
+#pragma unroll
+    for (int db = 0; db < 4; db++) {
+      i32x8 vf;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        i32x2 x = __builtin_amdgcn_ds_read_tr8_b64_v2i32((XDIT_LDS i32x2*)(vtile + r * 2 * ROW_BYTES + db * 32));
+        vf[2 * r] = x[0];
+        vf[2 * r + 1] = x[1];
+      }
+      oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[db], 0, 0, 0, 0, 0, 0);
+    }
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------
+  const float l_tot = sum_halves(l_part);
+  const float inv = sv / l_tot;
+  if (qrow < p.Sq) {
+    TO* optr = (TO*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        typedef __attribute__((ext_vector_type(4))) TO vec4;
+        f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                   oacc[db][4 * a + 3] * inv};
+        vec4 ov = __builtin_convertvector(o, vec4);
+        *(vec4*)(optr + 32 * db + 8 * a + 4 * hh) = ov;
+      }
+    if (p.lse != nullptr && hh == 0) {
+      p.lse[b * p.ls_b + h * p.ls_h + qrow] = (m_used * c - kPShift + fast_log2(l_tot)) * kLn2;
+    }
+  }
+}
+
+}  // namespace fp8path
+
+hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, hipStream_t stream) {
+  AttnParams q = p;
+  q.nq_tiles = (p.Sq + fp8path::kRowsPerBlock - 1) / fp8path::kRowsPerBlock;
+  q.total_tiles = p.B * p.H * q.nq_tiles;
+  q.tiles_per_xcd = (q.total_tiles + 7) / 8;
+  dim3 grid(q.tiles_per_xcd * 8);
+  if (out_is_fp16) hipLaunchKernelGGL((fp8path::attn_fwd_fp8_kernel<_Float16>), grid, dim3(256), 0, stream, q);
+  else hipLaunchKernelGGL((fp8path::attn_fwd_fp8_kernel<__bf16>), grid, dim3(256), 0, stream, q);
+  return hipGetLastError();
+}
+
+}  // namespace xdit

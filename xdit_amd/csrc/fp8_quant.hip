@@ -1,0 +1,140 @@
+// fp8 (OCP e4m3fn) quantiser with abs-max scaling for gfx950: the step in front of the fp8
+// attention kernel.  Restates per_tensor_quant (xfuser/core/distributed/attention_backend.py:606-615):
+//     scale = absmax(x) / 448 ;  y = fp8(x / scale) ;  descale = scale broadcast to (B, H)
+// with the abs-max taken over the whole tensor (`per_tensor`) or per (batch, head) slice, or a
+// caller-supplied static scale.  Four small launches on the caller's stream, two of which touch
+// the tensor: (1) clear the (B,H) abs-max buffer (a fill kernel, so the sequence can be captured
+// in a HIP graph), (2) abs-max reduction with one atomic max per workgroup, (3) scale and cast,
+// (4) turn the abs-max buffer into the descale values.  Both tensor passes are HBM-bound and read
+// 16 bytes per lane; the division is a true fp32 division so results match the reference's
+// `x / scale` bit for bit.
+#include "common.h"
+#include "launchers.h"
+
+namespace xdit {
+
+namespace quant {
+
+constexpr float kFp8Max = 448.0f;
+
+template <typename T> __device__ __forceinline__ void load8(const T* p, float (&x)[8]);
+template <> __device__ __forceinline__ void load8<float>(const float* p, float (&x)[8]) {
+  f32x4 a = ((const f32x4*)p)[0], b = ((const f32x4*)p)[1];
+  for (int i = 0; i < 4; i++) { x[i] = a[i]; x[4 + i] = b[i]; }
+}
+template <> __device__ __forceinline__ void load8<__bf16>(const __bf16* p, float (&x)[8]) {
+  bf16x8 v = *(const bf16x8*)p;
+  for (int i = 0; i < 8; i++) x[i] = (float)v[i];
+}
+template <> __device__ __forceinline__ void load8<_Float16>(const _Float16* p, float (&x)[8]) {
+  f16x8 v = *(const f16x8*)p;
+  for (int i = 0; i < 8; i++) x[i] = (float)v[i];
+}
+
+__global__ void fill_zero_kernel(float* p, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
+// grid = (blocks per slice, B*H); each thread walks 8-element chunks of its (b,h) slice.
+template <typename T>
+__global__ __launch_bounds__(256) void absmax_kernel(const QuantParams p) {
+  const int bh = blockIdx.y;
+  const int b = bh / p.H, h = bh - b * p.H;
+  const T* x = (const T*)p.x + b * p.xs_b + h * p.xs_h;
+  const int cpr = p.D >> 3;
+  const int64_t chunks = (int64_t)p.S * cpr;
+  float m = 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * 256) {
+    const int64_t s = i / cpr;
+    const int c = (int)(i - s * cpr);
+    float v[8];
+    load8<T>(x + s * p.xs_s + c * 8, v);
+#pragma unroll
+    for (int j = 0; j < 8; j++) m = fmaxf(m, fabsf(v[j]));  // fmaxf drops NaN operands
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  __shared__ float wm[4];
+  if ((threadIdx.x & 63) == 0) wm[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = fmaxf(fmaxf(wm[0], wm[1]), fmaxf(wm[2], wm[3]));
+    // non-negative floats order like their bit patterns
+    atomicMax((unsigned int*)(p.amax + (p.per_tensor ? 0 : bh)), __float_as_uint(m));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void cast_kernel(const QuantParams p) {
+  const int bh = blockIdx.y;
+  const int b = bh / p.H, h = bh - b * p.H;
+  const T* x = (const T*)p.x + b * p.xs_b + h * p.xs_h;
+  unsigned char* y = (unsigned char*)p.y + b * p.ys_b + h * p.ys_h;
+  float scale;
+  if (p.scale_in != nullptr) {
+    scale = *p.scale_in;
+  } else {
+    const float am = p.amax[p.per_tensor ? 0 : bh];
+    scale = am > 0.f ? am / kFp8Max : 1.0f;
+  }
+  const int cpr = p.D >> 3;
+  const int64_t chunks = (int64_t)p.S * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * 256) {
+    const int64_t s = i / cpr;
+    const int c = (int)(i - s * cpr);
+    float v[8];
+    load8<T>(x + s * p.xs_s + c * 8, v);
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = v[j] / scale;
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w0, true);
+    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], 0, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], w1, true);
+    i32x2 w = {w0, w1};
+    *(i32x2*)(y + s * p.ys_s + c * 8) = w;
+  }
+}
+
+// amax buffer -> descale values, for all B*H entries.
+__global__ void finalize_kernel(const QuantParams p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  // every thread reads its source before any thread overwrites entry 0 (single workgroup launch
+  // when per_tensor; otherwise each thread only touches its own entry)
+  float am = (p.scale_in != nullptr) ? 0.f : p.amax[p.per_tensor ? 0 : (i < n ? i : 0)];
+  __syncthreads();
+  if (i >= n) return;
+  float scale = (p.scale_in != nullptr) ? *p.scale_in : (am > 0.f ? am / kFp8Max : 1.0f);
+  p.descale[i] = scale;
+}
+
+template <typename T>
+static hipError_t run(const QuantParams& p, hipStream_t stream) {
+  const int BH = p.B * p.H;
+  const int64_t chunks = (int64_t)p.S * (p.D >> 3);
+  int per_slice = (int)((chunks + 256 * 8 - 1) / (256 * 8));  // ~8 chunks per thread
+  if (per_slice < 1) per_slice = 1;
+  if (per_slice > 2048) per_slice = 2048;
+  dim3 grid(per_slice, BH), block(256);
+  if (p.scale_in == nullptr) {
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((BH + 255) / 256), dim3(256), 0, stream, p.amax, BH);
+    hipLaunchKernelGGL((absmax_kernel<T>), grid, block, 0, stream, p);
+  }
+  hipLaunchKernelGGL((cast_kernel<T>), grid, block, 0, stream, p);
+  // per_tensor broadcasts entry 0: keep it to one workgroup so the barrier orders read/write
+  if (p.per_tensor && BH > 1024) return hipErrorInvalidValue;
+  const int fb = p.per_tensor ? BH : 256;
+  hipLaunchKernelGGL(finalize_kernel, dim3((BH + fb - 1) / fb), dim3(fb < 64 ? 64 : fb), 0, stream, p, BH);
+  return hipGetLastError();
+}
+
+}  // namespace quant
+
+hipError_t launch_fp8_quant(const QuantParams& p, int in_dtype, hipStream_t stream) {
+  if (in_dtype == 0) return quant::run<__bf16>(p, stream);
+  if (in_dtype == 1) return quant::run<_Float16>(p, stream);
+  if (in_dtype == 2) return quant::run<float>(p, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace xdit

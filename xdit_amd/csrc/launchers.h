@@ -24,10 +24,25 @@ struct MergeParams {
   int64_t rows;  // B * H * S
 };
 
+// Parameters of one fp8 quantiser call.  `amax` and `descale` are the same (B,H) fp32 buffer:
+// it holds the abs-max values between the passes and the descales at the end.
+struct QuantParams {
+  const void* x;
+  void* y;
+  float* amax;
+  float* descale;
+  const float* scale_in;  // optional static scale (one float); skips the abs-max pass
+  int64_t xs_b, xs_h, xs_s;
+  int64_t ys_b, ys_h, ys_s;
+  int B, H, S, D;
+  int per_tensor;
+};
+
 // dtype codes below are the C ABI's xdit_dtype values: 0 bf16, 1 fp16, 2 fp32, 3 fp8 e4m3fn.
 hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, hipStream_t stream);
 hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, hipStream_t stream);
 hipError_t launch_attn_fwd_f32(const AttnParams& p, int dtype, int D, hipStream_t stream);
+hipError_t launch_fp8_quant(const QuantParams& p, int in_dtype, hipStream_t stream);
 hipError_t launch_lse_merge(const MergeParams& p, int block_dtype, int final_dtype, hipStream_t stream);
 
 }  // namespace xdit

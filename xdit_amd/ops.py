@@ -153,3 +153,28 @@ def lse_merge(acc_out, acc_lse, block_out, block_lse, first=False, final_out=Non
     with torch.cuda.device(device):
         _lib.check(_lib.lib().xdit_lse_merge(ctypes.byref(a)))
     return acc_out, acc_lse
+
+
+def fp8_quant(x, per_tensor=False, scale=None):
+    """Abs-max fp8 quantiser on a logical BHSD tensor -> (y float8_e4m3fn BHSD-contiguous,
+    descale (B,H) fp32).  `per_tensor` takes one abs-max over the whole tensor (the reference's
+    per_tensor_quant); `scale` (a one-element fp32 tensor) is a static scale."""
+    device = x.device
+    _check4("x", x, device)
+    B, H, S, D = x.shape
+    y = torch.empty((B, H, S, D), dtype=torch.float8_e4m3fn, device=device)
+    descale = torch.empty((B, H), dtype=torch.float32, device=device)
+    a = _lib.QuantArgs()
+    a.struct_size = ctypes.sizeof(_lib.QuantArgs)
+    a.in_dtype = _code(x.dtype)
+    a.per_tensor = 1 if per_tensor else 0
+    a.B, a.H, a.D, a.S = B, H, D, S
+    a.x, a.y, a.descale = x.data_ptr(), y.data_ptr(), descale.data_ptr()
+    if scale is not None:
+        scale = scale.to(device=device, dtype=torch.float32).reshape(1).contiguous()
+        a.scale_in = scale.data_ptr()
+    a.x_stride, a.y_stride = _strides(x), _strides(y)
+    a.stream = _stream(device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().xdit_fp8_quant(ctypes.byref(a)))
+    return y, descale
