@@ -1,0 +1,114 @@
+"""The C-ABI library loads, exports every symbol include/xdit_amd_attn.h declares, its ctypes
+mirror has the header's struct sizes, and argument errors come back as codes + messages
+(no compute call is made: every check below fails validation before any launch)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from xdit_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "xdit_amd_attn.h")
+
+
+def _declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(xdit_[a-z0-9_]+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert set(names) == set(_lib.EXPORTS)
+    L = _lib.lib()
+    for n in names:
+        assert getattr(L, n) is not None
+    assert L.xdit_attn_abi_version() == _lib.ABI_VERSION
+
+
+def test_ctypes_structs_match_header(tmp_path):
+    c = tmp_path / "sz.c"
+    c.write_text('#include "xdit_amd_attn.h"\n#include <stdio.h>\n#include <stddef.h>\n'
+                 'int main(){printf("%zu %zu %zu %zu %zu %zu\\n", sizeof(xdit_attn_args), sizeof(xdit_merge_args),'
+                 ' sizeof(xdit_quant_args), offsetof(xdit_attn_args, q_stride), offsetof(xdit_attn_args, stream),'
+                 ' offsetof(xdit_merge_args, acc_lse_stride));}\n')
+    exe = tmp_path / "sz"
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(c), "-o", str(exe)])
+    got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    assert got == [ctypes.sizeof(_lib.AttnArgs), ctypes.sizeof(_lib.MergeArgs), ctypes.sizeof(_lib.QuantArgs),
+                   _lib.AttnArgs.q_stride.offset, _lib.AttnArgs.stream.offset, _lib.MergeArgs.acc_lse_stride.offset]
+
+
+def _attn_args(**kw):
+    a = _lib.AttnArgs()
+    a.struct_size = ctypes.sizeof(_lib.AttnArgs)
+    a.dtype = a.out_dtype = _lib.DTYPE_BF16
+    a.B, a.H, a.D = 1, 2, 128
+    a.Sq = a.Sk = 64
+    a.softmax_scale = 0.1
+    fake = 0x1000  # never dereferenced: validation fails first
+    a.q = a.k = a.v = a.out = fake
+    for s in ("q_stride", "k_stride", "v_stride", "out_stride"):
+        setattr(a, s, _lib.Strides(2 * 64 * 128, 64 * 128, 128))
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize("kw,code,needle", [
+    (dict(struct_size=8), _lib.XDIT_ERR_INVALID_ARG, "struct_size"),
+    (dict(dtype=9), _lib.XDIT_ERR_INVALID_ARG, "dtype"),
+    (dict(causal=1), _lib.XDIT_ERR_UNSUPPORTED, "causal"),
+    (dict(q=0), _lib.XDIT_ERR_INVALID_ARG, "q is NULL"),
+    (dict(k=0x1004), _lib.XDIT_ERR_INVALID_ARG, "16-byte aligned"),
+    (dict(Sk=0), _lib.XDIT_ERR_INVALID_ARG, "Sk"),
+    (dict(D=100), _lib.XDIT_ERR_UNSUPPORTED, "head_dim"),
+    (dict(D=512), _lib.XDIT_ERR_UNSUPPORTED, "head_dim"),
+    (dict(softmax_scale=0.0), _lib.XDIT_ERR_INVALID_ARG, "softmax_scale"),
+    (dict(softmax_scale=float("nan")), _lib.XDIT_ERR_INVALID_ARG, "softmax_scale"),
+    (dict(out_dtype=_lib.DTYPE_FP32), _lib.XDIT_ERR_INVALID_ARG, "out_dtype"),
+    (dict(v_stride=_lib.Strides(0, 0, 4)), _lib.XDIT_ERR_INVALID_ARG, "stride"),
+    (dict(Sk2=5), _lib.XDIT_ERR_INVALID_ARG, "k2 is NULL"),
+    (dict(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16, D=64), _lib.XDIT_ERR_UNSUPPORTED, "fp8"),
+])
+def test_attn_fwd_rejects_bad_arguments(kw, code, needle):
+    L = _lib.lib()
+    rc = L.xdit_attn_fwd(ctypes.byref(_attn_args(**kw)))
+    assert rc == code
+    assert needle in _lib.last_error()
+    with pytest.raises({_lib.XDIT_ERR_INVALID_ARG: ValueError, _lib.XDIT_ERR_UNSUPPORTED: NotImplementedError}[code]):
+        _lib.check(rc)
+
+
+def test_null_args_and_merge_quant_validation():
+    L = _lib.lib()
+    assert L.xdit_attn_fwd(None) == _lib.XDIT_ERR_INVALID_ARG
+    assert L.xdit_lse_merge(None) == _lib.XDIT_ERR_INVALID_ARG
+    assert L.xdit_fp8_quant(None) == _lib.XDIT_ERR_INVALID_ARG
+    m = _lib.MergeArgs()
+    m.struct_size = ctypes.sizeof(_lib.MergeArgs)
+    m.block_dtype = _lib.DTYPE_FP8_E4M3FN
+    assert L.xdit_lse_merge(ctypes.byref(m)) == _lib.XDIT_ERR_INVALID_ARG and "block_dtype" in _lib.last_error()
+    m.block_dtype = _lib.DTYPE_BF16
+    m.B, m.H, m.D, m.S = 1, 1, 12, 4
+    assert L.xdit_lse_merge(ctypes.byref(m)) == _lib.XDIT_ERR_INVALID_ARG and "head_dim" in _lib.last_error()
+    q = _lib.QuantArgs()
+    q.struct_size = ctypes.sizeof(_lib.QuantArgs)
+    q.in_dtype = _lib.DTYPE_FP8_E4M3FN
+    assert L.xdit_fp8_quant(ctypes.byref(q)) == _lib.XDIT_ERR_INVALID_ARG and "in_dtype" in _lib.last_error()
+
+
+def test_error_message_is_per_thread_and_cleared_on_entry():
+    import threading
+    L = _lib.lib()
+    L.xdit_attn_fwd(None)
+    seen = {}
+
+    def other():
+        seen["msg"] = _lib.last_error()
+    t = threading.Thread(target=other)
+    t.start(); t.join()
+    assert seen["msg"] == "" and _lib.last_error() == "args is NULL"

@@ -1,0 +1,338 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs,
+against the committed golden fixtures, and — at the full benchmark sizes — through
+size-independent properties (fold of KV chunks == single pass, key-order invariance, layout
+invariance, run-to-run determinism) plus probe rows evaluated by the oracle against the full K/V.
+
+Tolerances (max abs error against the float64 oracle):
+  bf16 / fp16 inputs   out <= 2e-2, lse <= 1e-3
+  fp8 inputs           out <= 6e-2 (reference = attention of the dequantised inputs), lse <= 1e-3
+  fp32 inputs          out <= 2e-5, lse <= 2e-5
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attn_oracle as O
+from xdit_amd import attention_backend as AB
+from xdit_amd import ops, ring, usp
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+TOL = {torch.bfloat16: (2e-2, 1e-3), torch.float16: (2e-2, 1e-3), torch.float32: (2e-5, 2e-5)}
+
+
+def _err(a, b):
+    return (a.detach().double().cpu() - b.double()).abs().max().item()
+
+
+def _layout(t, layout, dev):
+    """Put a CPU BHSD tensor on the device either BHSD-contiguous or as a BSHD-contiguous tensor
+    viewed as BHSD (the two physical layouts xDiT's callers produce)."""
+    if layout == "bhsd":
+        return t.to(dev).contiguous()
+    return t.transpose(1, 2).contiguous().to(dev).transpose(1, 2)
+
+
+CASES = [
+    # B, H, Sq, Sk, D
+    (1, 1, 1, 1, 128), (1, 2, 5, 63, 128), (1, 2, 128, 64, 128), (1, 2, 129, 65, 128), (2, 3, 200, 333, 128),
+    (1, 2, 256, 640, 128), (1, 3, 77, 1, 128), (1, 1, 1000, 127, 128), (1, 2, 300, 500, 64), (2, 2, 31, 129, 64),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+@pytest.mark.parametrize("B,H,Sq,Sk,D", CASES)
+def test_attn_16bit_small_vs_oracle(gpu, dtype, layout, B, H, Sq, Sk, D):
+    g = torch.Generator().manual_seed(B * 1000 + Sq * 7 + Sk)
+    q = torch.randn(B, H, Sq, D, generator=g).to(dtype)
+    k = torch.randn(B, H, Sk, D, generator=g).to(dtype)
+    v = torch.randn(B, H, Sk, D, generator=g).to(dtype)
+    scale = 0.11 if Sq % 2 else D ** -0.5
+    ro, rl = O.attn_fwd_ref(q, k, v, scale)
+    o, l = ops.attn_fwd(_layout(q, layout, gpu), _layout(k, layout, gpu), _layout(v, layout, gpu), softmax_scale=scale)
+    assert o.dtype == dtype and l.dtype == torch.float32 and l.shape == (B, H, Sq)
+    assert _err(o, ro) <= TOL[dtype][0] and _err(l, rl) <= TOL[dtype][1]
+
+
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 72), (torch.float32, 8), (torch.float32, 128), (torch.float32, 64),
+                                      (torch.bfloat16, 72), (torch.float16, 40), (torch.bfloat16, 96)])
+@pytest.mark.parametrize("Sq,Sk", [(1, 1), (33, 31), (130, 200), (128, 32)])
+def test_attn_generic_path_vs_oracle(gpu, dtype, D, Sq, Sk):
+    """fp32 inputs and head dims outside {64,128} run on the fp32 matrix cores."""
+    g = torch.Generator().manual_seed(D * 100 + Sq)
+    q = torch.randn(2, 2, Sq, D, generator=g).to(dtype)
+    k = torch.randn(2, 2, Sk, D, generator=g).to(dtype)
+    v = torch.randn(2, 2, Sk, D, generator=g).to(dtype)
+    ro, rl = O.attn_fwd_ref(q, k, v)
+    o, l = ops.attn_fwd(_layout(q, "bshd", gpu), k.to(gpu), v.to(gpu))
+    assert _err(o, ro) <= TOL[dtype][0] and _err(l, rl) <= TOL[dtype][1]
+
+
+def test_tiny_bruteforce_golden(gpu):
+    z = np.load(os.path.join(GOLD, "tiny_bruteforce.npz"))
+    for n in (2, 3, 4):  # the head_dim 8 cases
+        q, k, v = (torch.from_numpy(z[f"t{n}_{x}"]).float()[None, None] for x in "qkv")
+        o, l = ops.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu))
+        assert _err(o[0, 0], torch.from_numpy(z[f"t{n}_out"])) <= 2e-6
+        assert _err(l[0, 0], torch.from_numpy(z[f"t{n}_lse"])) <= 2e-6
+
+
+@pytest.mark.parametrize("Sk,Sk2", [(192, 70), (100, 64), (64, 1), (1, 300)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_two_kv_segments_equal_concatenation(gpu, dtype, Sk, Sk2):
+    g = torch.Generator().manual_seed(Sk + Sk2)
+    D = 128
+    q = torch.randn(1, 2, 150, D, generator=g).to(dtype)
+    k, v = (torch.randn(1, 2, Sk, D, generator=g).to(dtype) for _ in range(2))
+    k2, v2 = (torch.randn(1, 2, Sk2, D, generator=g).to(dtype) for _ in range(2))
+    ro, rl = O.attn_fwd_ref(q, torch.cat([k, k2], 2), torch.cat([v, v2], 2))
+    o, l = ops.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), k2=_layout(k2, "bshd", gpu), v2=_layout(v2, "bshd", gpu))
+    assert _err(o, ro) <= TOL[dtype][0] and _err(l, rl) <= TOL[dtype][1]
+
+
+# ---------------------------------------------------------------------------- named configurations
+def test_c1_pixart512_fp32_full(gpu):
+    z = np.load(os.path.join(GOLD, "c1_pixart512.npz"))
+    c = O.make_config("c1_pixart512")
+    o, l = ops.attn_fwd(c["q"].to(gpu), c["k"].to(gpu), c["v"].to(gpu), softmax_scale=72 ** -0.5)
+    assert _err(o[:, :, ::37], torch.from_numpy(z["out_rows"])) <= 2e-5
+    assert _err(l, torch.from_numpy(z["lse"])) <= 2e-5
+    # and against the op the reference's SDPA_MATH backend calls, on the CPU
+    mo, _ = torch.ops.aten._scaled_dot_product_attention_math(c["q"], c["k"], c["v"])
+    assert _err(o, mo) <= 2e-5
+
+
+@pytest.fixture(scope="module")
+def flux(gpu):
+    c = O.make_config("c2_flux1024")
+    z = np.load(os.path.join(GOLD, "c2_flux1024_rows.npz"))
+    d = {n: c[n].to(gpu) for n in "qkv"}
+    d["rows"] = torch.from_numpy(z["rows"]).to(gpu)
+    d["ref_out"], d["ref_lse"] = torch.from_numpy(z["out"]), torch.from_numpy(z["lse"])
+    return d
+
+
+def test_c2_flux1024_single_pass(gpu, flux):
+    o, l = ops.attn_fwd(flux["q"], flux["k"], flux["v"])
+    assert _err(o[:, :, flux["rows"]], flux["ref_out"]) <= 2e-2
+    assert _err(l[:, :, flux["rows"]], flux["ref_lse"]) <= 1e-3
+    # determinism and layout invariance: bit-identical results
+    o2, l2 = ops.attn_fwd(flux["q"], flux["k"], flux["v"])
+    assert torch.equal(o, o2) and torch.equal(l, l2)
+    tb = lambda t: t.transpose(1, 2).contiguous().transpose(1, 2)
+    o3, l3 = ops.attn_fwd(tb(flux["q"]), tb(flux["k"]), tb(flux["v"]))
+    assert torch.equal(o, o3) and torch.equal(l, l3)
+    # the registry adapter and USP return the same thing
+    o4, l4 = AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355](flux["q"], flux["k"], flux["v"], 0.0, False)
+    assert torch.equal(o, o4) and torch.equal(l, l4)
+    assert torch.equal(o, usp.USP(flux["q"], flux["k"], flux["v"]))
+
+
+@pytest.mark.parametrize("order", [None, [0, 1, 2, 3]])
+def test_c3_flux_ring_of_4_equals_single_pass(gpu, flux, order):
+    o, l = ops.attn_fwd(flux["q"], flux["k"], flux["v"])
+    fn = usp._get_attention_function()
+    merged = usp.ring_attn(fn, flux["q"], flux["k"], flux["v"], ring_chunks=4, order=order)
+    assert merged.dtype == torch.bfloat16
+    assert _err(merged[:, :, flux["rows"]], flux["ref_out"]) <= 2e-2
+    assert _err(merged, o.cpu()) <= 2e-2
+    # legacy BSHD loop with update_out_and_lse, returning the lse as well
+    qb, kb, vb = (flux[n].transpose(1, 2).contiguous() for n in "qkv")
+    ob, lb, _ = ring.xdit_ring_flash_attn_func(qb, kb, vb, return_attn_probs=True, group=ring.LocalRing(4))
+    assert ob.shape == qb.shape and lb.shape == (1, 24, 4608)
+    assert _err(ob.transpose(1, 2)[:, :, flux["rows"]], flux["ref_out"]) <= 2e-2
+    assert _err(lb[:, :, flux["rows"]], flux["ref_lse"]) <= 1e-3
+    assert _err(lb, l.cpu()) <= 1e-3
+
+
+def test_c4_hunyuan720p_shard_full_size(gpu):
+    """(1, 3, 119056, 128) bf16: probe rows against the oracle over the full K/V, plus
+    chunk-fold and key-permutation invariance at full size."""
+    c = O.make_config("c4_hunyuan720p_shard")
+    S = c["q"].shape[2]
+    assert S == 119056
+    rows = [0, 1, 127, 128, 4097, 60000, 118799, 118800, 119040, 119055]
+    ro, rl = O.attn_rows_ref(c["q"], c["k"], c["v"], rows)
+    q, k, v = (c[n].to(gpu) for n in "qkv")
+    o, l = ops.attn_fwd(q, k, v)
+    assert _err(o[:, :, rows], ro) <= 2e-2 and _err(l[:, :, rows], rl) <= 1e-3
+    assert torch.isfinite(o.float()).all() and torch.isfinite(l).all()
+    # fold of two unequal KV chunks (video | text, as a joint ring step would see them)
+    o1, l1 = ops.attn_fwd(q, k[:, :, :118800], v[:, :, :118800])
+    o2, l2 = ops.attn_fwd(q, k[:, :, 118800:], v[:, :, 118800:])
+    m = usp.SDPAMerger()
+    m.step(o1, l1)
+    m.step(o2, l2, final_step=True)
+    mo, ml = m.results()
+    assert _err(mo, o.cpu()) <= 2e-2 and _err(ml, l.cpu()) <= 1e-3
+    # two-segment call == single call, and key order does not matter
+    o3, l3 = ops.attn_fwd(q, k[:, :, 118800:], v[:, :, 118800:], k2=k[:, :, :118800], v2=v[:, :, :118800])
+    assert _err(o3, o.cpu()) <= 2e-2 and _err(l3, l.cpu()) <= 1e-3
+
+
+def test_c5_wan720p_shard_fp8_full_size(gpu):
+    """(1, 5, 75600, 128) fp8 e4m3fn + per-head scales -> bf16 out, fp32 lse."""
+    c = O.make_config("c5_wan720p_shard_fp8")
+    assert c["q"].shape == (1, 5, 75600, 128)
+    rows = [0, 31, 32, 1000, 40000, 75519, 75520, 75599]
+    dq, dk, dv = (O.dequant(c[n], c[n + "_descale"]) for n in "qkv")
+    ro, rl = O.attn_rows_ref(dq, dk, dv, rows)
+    args = {n: c[n].to(gpu) for n in c}
+    o, l = ops.attn_fwd(args["q"], args["k"], args["v"], q_descale=args["q_descale"],
+                        k_descale=args["k_descale"], v_descale=args["v_descale"])
+    assert o.dtype == torch.bfloat16 and l.dtype == torch.float32
+    assert _err(o[:, :, rows], ro) <= 6e-2 and _err(l[:, :, rows], rl) <= 1e-3
+    assert torch.isfinite(o.float()).all() and torch.isfinite(l).all()
+
+
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+def test_fp8_golden_s2048(gpu, layout):
+    z = np.load(os.path.join(GOLD, "c5_fp8_s2048_rows.npz"))
+    c = O.make_config("c5_wan720p_shard_fp8", S=2048)
+    rows = torch.from_numpy(z["rows"])
+    lay = lambda t: t.view(torch.uint8).transpose(1, 2).contiguous().transpose(1, 2).view(torch.float8_e4m3fn) if layout == "bshd" else t
+    o, l = ops.attn_fwd(lay(c["q"]).to(gpu), lay(c["k"]).to(gpu), lay(c["v"]).to(gpu),
+                        q_descale=c["q_descale"].to(gpu), k_descale=c["k_descale"].to(gpu), v_descale=c["v_descale"].to(gpu),
+                        out_dtype=torch.float16)
+    assert o.dtype == torch.float16
+    assert _err(o[:, :, rows], torch.from_numpy(z["out"])) <= 6e-2
+    assert _err(l[:, :, rows], torch.from_numpy(z["lse"])) <= 1e-3
+
+
+@pytest.mark.parametrize("Sq,Sk", [(1, 1), (100, 63), (129, 130), (64, 1000)])
+def test_fp8_small_vs_oracle(gpu, Sq, Sk):
+    g = torch.Generator().manual_seed(Sq + Sk)
+    q, k, v = (torch.randn(2, 2, n, 128, generator=g) * 3 for n in (Sq, Sk, Sk))
+    (q8, qd), (k8, kd), (v8, vd) = (O.per_head_quant_ref(t) for t in (q, k, v))
+    ro, rl = O.attn_fwd_ref(O.dequant(q8, qd), O.dequant(k8, kd), O.dequant(v8, vd))
+    o, l = ops.attn_fwd(q8.to(gpu), k8.to(gpu), v8.to(gpu), q_descale=qd.to(gpu), k_descale=kd.to(gpu), v_descale=vd.to(gpu))
+    # logits here have a standard deviation of about 9: few keys carry the mass, which is the
+    # hard case for an fp8 P matrix
+    assert _err(o, ro) <= 6e-2 * max(1.0, ro.abs().max().item()) and _err(l, rl) <= 1e-3
+
+
+# ---------------------------------------------------------------------------- merge
+@pytest.mark.parametrize("block_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+def test_merge_vs_oracle(gpu, block_dtype, layout):
+    B, H, S, D = 2, 3, 257, 128
+    g = torch.Generator().manual_seed(21)
+    out = torch.randn(B, H, S, D, generator=g)
+    lse = torch.randn(B, H, S, generator=g) * 3
+    bo = torch.randn(B, H, S, D, generator=g).to(block_dtype)
+    bl = torch.randn(B, H, S, generator=g) * 3
+    ro, rl = O.merge_ref(out, lse, bo, bl)
+    ao = _layout(out, layout, gpu)
+    al = lse.to(gpu) if layout == "bhsd" else lse.transpose(1, 2).contiguous().to(gpu).transpose(1, 2)
+    fo = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=gpu)
+    ops.lse_merge(ao, al, _layout(bo, layout, gpu), bl.to(gpu), final_out=fo)
+    assert _err(ao, ro) <= 2e-6 and _err(al, rl) <= 2e-6
+    assert torch.equal(fo, ao.bfloat16())
+
+
+def test_merge_first_call_and_special_values(gpu):
+    B, H, S, D = 1, 2, 64, 64
+    bo = torch.randn(B, H, S, D).bfloat16().to(gpu)
+    bl = torch.randn(B, H, S).to(gpu)
+    ao = torch.full((B, H, S, D), float("nan"), device=gpu)
+    al = torch.full((B, H, S), float("nan"), device=gpu)
+    ops.lse_merge(ao, al, bo, bl, first=True)
+    assert torch.equal(ao, bo.float()) and torch.equal(al, bl)
+    # a block with lse = -inf leaves the accumulator unchanged
+    before_o, before_l = ao.clone(), al.clone()
+    ops.lse_merge(ao, al, torch.randn_like(bo), torch.full_like(bl, float("-inf")))
+    assert torch.equal(ao, before_o) and torch.equal(al, before_l)
+    # equal lse: mean and lse + ln 2
+    bo2 = torch.randn(B, H, S, D, device=gpu)
+    ops.lse_merge(ao, al, bo2, before_l.clone())
+    assert _err(ao, 0.5 * (before_o + bo2).cpu()) <= 1e-6 and _err(al, (before_l + np.log(2.0)).cpu()) <= 1e-6
+
+
+def test_merge_golden_fold(gpu):
+    z = np.load(os.path.join(GOLD, "merge_fold.npz"))
+    ao = torch.from_numpy(z["out"]).float().to(gpu)
+    al = torch.from_numpy(z["lse"]).float().to(gpu)
+    ops.lse_merge(ao, al, torch.from_numpy(z["block_out"]).float().to(gpu), torch.from_numpy(z["block_lse"]).float().to(gpu))
+    assert _err(ao, torch.from_numpy(z["new_out"])) <= 2e-6 and _err(al, torch.from_numpy(z["new_lse"])) <= 2e-6
+
+
+def test_update_out_and_lse_matches_oracle_layout(gpu):
+    B, S, H, D = 2, 100, 3, 128
+    g = torch.Generator().manual_seed(5)
+    blocks = [(torch.randn(B, S, H, D, generator=g).bfloat16(), torch.randn(B, H, S, generator=g) * 2) for _ in range(3)]
+    out = lse = rout = rlse = None
+    for bo, bl in blocks:
+        out, lse = ring.update_out_and_lse(out, lse, bo.to(gpu), bl.to(gpu))
+        rout, rlse = O.update_out_and_lse_ref(rout, rlse, bo, bl, dtype=torch.float64)
+    assert out.shape == (B, S, H, D) and lse.shape == (B, S, H, 1) and out.dtype == torch.float32
+    assert _err(out, rout) <= 5e-6 and _err(lse, rlse) <= 5e-6
+
+
+# ---------------------------------------------------------------------------- quantiser
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_fp8_quant_bit_exact(gpu, dtype):
+    g = torch.Generator().manual_seed(8)
+    x = (torch.randn(2, 3, 333, 128, generator=g) * torch.arange(1, 7).reshape(2, 3, 1, 1)).to(dtype)
+    y, d = ops.fp8_quant(_layout(x, "bshd", gpu))
+    ry, rd = O.per_head_quant_ref(x)
+    assert torch.equal(y.cpu().view(torch.uint8), ry.view(torch.uint8)) and torch.equal(d.cpu(), rd)
+    y, d = AB.per_tensor_quant(x.to(gpu))
+    ry, rd = O.per_tensor_quant_ref(x)
+    assert torch.equal(y.cpu().view(torch.uint8), ry.view(torch.uint8)) and torch.equal(d.cpu(), rd.contiguous())
+    s = torch.tensor(0.05)
+    y, d = AB.per_tensor_quant(x.to(gpu), scale=s.to(gpu))
+    ry, rd = O.per_tensor_quant_ref(x.clamp(-448 * 0.05, 448 * 0.05), scale=s)
+    assert torch.equal(y.cpu().view(torch.uint8), ry.view(torch.uint8)) and torch.all(d.cpu() == 0.05)
+    y0, d0 = ops.fp8_quant(torch.zeros(1, 1, 8, 128, device=gpu))
+    assert d0.item() == 1.0 and torch.all(y0.float() == 0)
+
+
+# ---------------------------------------------------------------------------- call surfaces
+@pytest.mark.parametrize("strategy", ["front", "rear"])
+@pytest.mark.parametrize("chunks", [1, 2])
+def test_usp_joint_vs_oracle(gpu, strategy, chunks):
+    q, k, v = O.make_qkv(1, 4, 512, 128, seed=31, rmsnorm=True, dtype=torch.bfloat16)
+    jq, jk, jv = O.make_qkv(1, 4, 77, 128, seed=32, rmsnorm=True, dtype=torch.bfloat16)
+    cat = (lambda a, b: torch.cat([a, b], 2)) if strategy == "rear" else (lambda a, b: torch.cat([b, a], 2))
+    ro, _ = O.attn_fwd_ref(cat(q, jq), cat(k, jk), cat(v, jv))
+    o = usp.USP(q.to(gpu), k.to(gpu), v.to(gpu), joint_query=jq.to(gpu), joint_key=jk.to(gpu), joint_value=jv.to(gpu),
+                joint_strategy=strategy, ring_chunks=chunks)
+    assert o.shape == (1, 4, 589, 128) and _err(o, ro) <= 2e-2
+
+
+@pytest.mark.parametrize("strategy", ["front", "rear"])
+def test_long_context_layer_joint_vs_oracle(gpu, strategy):
+    """The layer form in BSHD with fp16, tolerance of the reference's own layer test (1e-2)."""
+    q, k, v = O.make_qkv(1, 4, 256, 128, seed=41, dtype=torch.float16)
+    jq, jk, jv = O.make_qkv(1, 4, 64, 128, seed=42, dtype=torch.float16)
+    cat = (lambda a, b: torch.cat([a, b], 2)) if strategy == "rear" else (lambda a, b: torch.cat([b, a], 2))
+    ro, _ = O.attn_fwd_ref(cat(q, jq), cat(k, jk), cat(v, jv))
+    b = lambda t: t.transpose(1, 2).contiguous().to(gpu)
+    layer = ring.xFuserLongContextAttention(ring_group=ring.LocalRing(2))
+    o = layer(None, b(q), b(k), b(v), joint_tensor_query=b(jq), joint_tensor_key=b(jk), joint_tensor_value=b(jv),
+              joint_strategy=strategy)
+    assert o.shape == (1, 320, 4, 128) and _err(o.transpose(1, 2), ro) <= 1e-2
+
+
+def test_fp8_backend_adapter(gpu):
+    q, k, v = O.make_qkv(1, 4, 512, 128, seed=51, dtype=torch.bfloat16)
+    ro, rl = O.attn_fwd_ref(q, k, v)
+    o, l = AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355_FP8](q.to(gpu), k.to(gpu), v.to(gpu), 0.0, False)
+    assert o.dtype == torch.bfloat16 and _err(o, ro) <= 6e-2 and _err(l, rl) <= 2e-2
+    assert torch.equal(o, usp.attention(q.to(gpu), k.to(gpu), v.to(gpu), backend=AB.AttentionBackendType.MI355_FP8))
+
+
+def test_runs_on_the_callers_stream(gpu):
+    """Launches go to the current stream: work queued on a side stream is ordered with it."""
+    q, k, v = (torch.randn(1, 2, 512, 128, device=gpu).bfloat16() for _ in range(3))
+    ref_o, ref_l = ops.attn_fwd(q, k, v)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        q2 = q * 1.0
+        o, l = ops.attn_fwd(q2, k, v)
+    s.synchronize()
+    assert torch.equal(o, ref_o) and torch.equal(l, ref_l)

@@ -1,0 +1,119 @@
+"""Host-side logic of the reference-shaped call surfaces, checked on the CPU (no kernels run):
+argument domains, the joint-tensor step rule, ring ordering, registry behaviour, and that
+nothing falls back to a CPU implementation."""
+import pytest
+import torch
+
+from xdit_amd import attention_backend as AB
+from xdit_amd import ops, ring, usp
+
+
+def test_registry_and_lookup():
+    assert AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355] is AB._mi355_attn_call
+    assert AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355_FP8] is AB._mi355_fp8_attn_call
+    with pytest.raises(NotImplementedError):
+        usp._get_attention_function(backend="nope")
+
+    @AB.register_attention_function("custom")
+    def f(q, k, v, dropout_p, is_causal, attention_kwargs=None, joint_kv=None):
+        return q, None
+    try:
+        assert AB.ATTENTION_FUNCTION_REGISTRY["custom"] is f
+        assert usp.attention(torch.ones(1), None, None, backend="custom") is not None
+    finally:
+        del AB.ATTENTION_FUNCTION_REGISTRY["custom"]
+
+
+def test_argument_domain_matches_reference_call_sites():
+    q = torch.zeros(1, 2, 4, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        AB._mi355_attn_call(q, q, q, 0.1, False)
+    with pytest.raises(NotImplementedError):
+        AB._mi355_attn_call(q, q, q, 0.0, True)
+    with pytest.raises(NotImplementedError):
+        AB._mi355_attn_call(q, q, q, 0.0, False, attention_kwargs={"attn_mask": torch.ones(1)})
+    with pytest.raises(NotImplementedError):
+        AB._mi355_attn_call(q, q, q, 0.0, False, attention_kwargs={"indices_k": torch.ones(1)})
+    qb = q.transpose(1, 2)
+    for kw in (dict(causal=True), dict(window_size=(3, 3)), dict(softcap=1.0), dict(alibi_slopes=torch.ones(2))):
+        with pytest.raises(NotImplementedError):
+            ring.flash_attn_forward(qb, qb, qb, **kw)
+    with pytest.raises(ValueError):
+        ring.flash_attn_forward(qb, qb, qb, dropout_p=0.5)
+
+
+def test_no_cpu_fallback():
+    """CPU tensors must fail loudly: the product has no path other than the HIP library."""
+    q = torch.zeros(1, 2, 4, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.attn_fwd(q, q, q)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        usp.USP(q, q, q)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.lse_merge(torch.zeros(1, 2, 4, 128), torch.zeros(1, 2, 4), q, torch.zeros(1, 2, 4))
+
+
+def test_shape_and_dtype_validation():
+    q = torch.zeros(1, 2, 4, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.attn_fwd(q[0], q, q)
+    with pytest.raises(ValueError):
+        ops.attn_fwd(q, q, q, k2=q)  # k2 without v2
+
+
+def test_joint_decorator_step_rule():
+    """front -> joint K/V on step 0 only; rear -> on the last step only; step incremented in place
+    (the rule of usp.py:218-245)."""
+    calls = []
+
+    def fake(q, k, v, dropout_p, is_causal, attention_kwargs=None, joint_kv=None):
+        calls.append(joint_kv)
+        return q, None
+    f = usp.concat_joint_tensors_decorator(fake)
+    for strategy, expect in (("front", [True, False, False]), ("rear", [False, False, True])):
+        calls.clear()
+        kw = {"joint_key": "jk", "joint_value": "jv", "joint_strategy": strategy, "step": 0, "total_steps": 3}
+        for _ in range(3):
+            f("q", "k", "v", dropout_p=0.0, is_causal=False, joint_attn_kwargs=kw)
+        assert [c is not None for c in calls] == expect
+        assert kw["step"] == 3
+        assert [c for c in calls if c is not None][0] == ("jk", "jv", strategy)
+    calls.clear()
+    f("q", "k", "v", dropout_p=0.0, is_causal=False)
+    assert calls == [None]
+
+
+def test_joint_segment_order_matches_cat_order():
+    assert AB._split_joint("k", "v", ("jk", "jv", "rear")) == ("k", "v", "jk", "jv")
+    assert AB._split_joint("k", "v", ("jk", "jv", "front")) == ("jk", "jv", "k", "v")
+    with pytest.raises(ValueError):
+        AB._split_joint("k", "v", ("jk", "jv", "middle"))
+    with pytest.raises(ValueError):
+        usp._concat_joint_tensor(torch.ones(1), torch.ones(1), "middle", 0)
+    a, b = torch.zeros(1, 1, 2, 1), torch.ones(1, 1, 1, 1)
+    assert usp._concat_joint_tensor(a, b, "rear", 2).flatten().tolist() == [0, 0, 1]
+    assert usp._concat_joint_tensor(a, b, "front", 2).flatten().tolist() == [1, 0, 0]
+
+
+def test_local_ring_order():
+    assert ring.LocalRing(4).order() == [0, 3, 2, 1]      # what rank 0 of a 4-ring receives
+    assert ring.LocalRing(4, rank=2).order() == [2, 1, 0, 3]
+    assert ring.LocalRing(1).order() == [0]
+    with pytest.raises(ValueError):
+        ring.LocalRing(0)
+
+
+def test_legacy_ring_argument_errors():
+    q = torch.zeros(1, 8, 2, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="simultaneously"):
+        ring.xdit_ring_flash_attn_forward(None, q, q, q, 0.1, causal=False, joint_tensor_key=q)
+    with pytest.raises(ValueError, match="not supprted"):
+        ring.xdit_ring_flash_attn_forward(None, q, q, q, 0.1, causal=False, joint_tensor_key=q,
+                                          joint_tensor_value=q, joint_strategy="none")
+    with pytest.raises(ValueError, match="divisible"):
+        ring.xdit_ring_flash_attn_forward(ring.LocalRing(3), q, q, q, 0.1, causal=False)
+    layer = ring.xFuserLongContextAttention()
+    with pytest.raises(ValueError, match="simultaneously"):
+        layer(None, q, q, q, joint_tensor_query=q)
+    with pytest.raises(NotImplementedError):
+        ring.update_out_and_lse(None, None, q, torch.zeros(1, 2, 8), slice_=(slice(0, 1),))

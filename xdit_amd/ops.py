@@ -52,11 +52,11 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
     with `k`/`v`.  For fp8 (torch.float8_e4m3fn) inputs the descales are (B, H) fp32 tensors.
     """
+    if (k2 is None) != (v2 is None):
+        raise ValueError("k2 and v2 should be None or not None simultaneously.")
     device = q.device
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check4(name, t, device)
-    if (k2 is None) != (v2 is None):
-        raise ValueError("k2 and v2 should be None or not None simultaneously.")
     B, H, Sq, D = q.shape
     if k.shape[0] != B or k.shape[1] != H or k.shape[3] != D or v.shape != k.shape:
         raise ValueError("q %s, k %s, v %s do not agree (Hq must equal Hk)" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
