@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
+
+A "step" is one call of the joint-attention forward on the Flux-1024 shape
+(B=1, H=24, S=4608 = 512 text + 4096 image tokens, D=128, bf16, non-causal, BHSD-contiguous,
+q/k per-head RMSNorm'd), inputs resident in HBM.  Prints ONE JSON line:
+  value        TFLOP/s of the step (algorithmic FLOPs 4*B*H*Sq*Sk*D over wall-clock per step)
+  ms_per_step  wall-clock per call over exactly K calls, synchronised on both sides
+  roofline     the same kernel's HIP-event average launch duration against the dense bf16 MFMA peak
+  cpu_baseline torch's CPU scaled_dot_product_attention (what the reference's SDPA adapter calls,
+               xfuser/core/distributed/attention_backend.py:499-501) on a bounded sample of the
+               same workload, timed on this host's cores
+  also         the other named shapes: HunyuanVideo-720p head shard (bf16), Wan2.1 720p head
+               shard (fp8), the 4-chunk ring with its fp32 merges, the merge kernel's GB/s
+Everything runs on one GPU; --gpus above 1 is refused (this build has no multi-GPU path).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def make_inputs(B, H, S, D, seed, device, rmsnorm=True, dtype=torch.bfloat16):
+    """Synthetic q, k, v ~ N(0,1) (BHSD); q and k get a per-head RMSNorm over head_dim with a gain
+    vector ~ U(0.8, 1.2), as a DiT block's norm_q / norm_k produce."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    def n():
+        return torch.randn((B, H, S, D), generator=g, dtype=torch.float32)
+    q, k, v = n(), n(), n()
+    if rmsnorm:
+        gq = 0.8 + 0.4 * torch.rand(D, generator=g)
+        gk = 0.8 + 0.4 * torch.rand(D, generator=g)
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6) * gq
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + 1e-6) * gk
+    return q.to(dtype).to(device), k.to(dtype).to(device), v.to(dtype).to(device)
+
+
+def time_calls(fn, steps, warmup):
+    """(wall ms per call, HIP-event ms per call) over exactly `steps` calls."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+
+def attn_flops(B, H, Sq, Sk, D):
+    return 4.0 * B * H * Sq * Sk * D
+
+
+def cpu_baseline(q, k, v, budget_s=12.0):
+    """The reference's CPU SDPA path on the same Flux-1024 tensors (all heads, fp32), repeated
+    for about `budget_s` seconds of CPU work; reports the median run."""
+    from oracle import attn_oracle as O   # the checker/baseline module; never used by the GPU leg
+    B, H, S, D = q.shape
+    qc, kc, vc = (t.float().cpu().contiguous() for t in (q, k, v))
+    O.sdpa_cpu(qc[:, :1], kc[:, :1], vc[:, :1])  # warm the thread pool
+    times = []
+    t_start = time.perf_counter()
+    while True:
+        t0 = time.perf_counter()
+        O.sdpa_cpu(qc, kc, vc)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_start > budget_s or len(times) >= 200:
+            break
+    t = sorted(times)[len(times) // 2]
+    return {
+        "value": round(attn_flops(B, H, S, S, D) / t / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "torch CPU scaled_dot_product_attention (the call inside the reference's SDPA adapter), fp32 copies of "
+                  "the same Flux-1024 tensors (B=1, H=%d, S=%d, D=%d), median of %d full-shape runs over %.1f s, "
+                  "%.3f s per run; host has %d logical CPUs, torch uses %d threads"
+                  % (H, S, D, len(times), time.perf_counter() - t_start, t, os.cpu_count(), torch.get_num_threads()),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof byte counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives / sharding code); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    from xdit_amd import ops, ring, usp  # loads the HIP library; raises if it is not built
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, H, S, D = 1, 24, 4608, 128
+    q, k, v = make_inputs(B, H, S, D, 1002, dev)
+    out = torch.empty_like(q)
+
+    def step():
+        ops.attn_fwd(q, k, v, out=out)
+
+    wall_ms, ev_ms = time_calls(step, args.steps, args.warmup)
+    flops = attn_flops(B, H, S, S, D)
+    tflops = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (ev_ms * 1e-3) / 1e12
+
+    result = {
+        "metric": "joint-attn fwd ms/call + TFLOP/s (% MFMA peak) at Flux-1024 and HV-720p shard",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "c2_flux1024: joint attention forward (out, lse), B=1 H=24 S=4608 (512 text + 4096 image) D=128, "
+                        "bf16, non-causal, BHSD-contiguous, RMSNorm'd q/k, single pass",
+            "flops_per_step": flops,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(achieved, 2),
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+            "traffic": None,
+            "kernel": "attn_fwd_16_kernel<bf16,128>",
+            "kernel_ms": round(ev_ms, 5),
+        },
+    }
+
+    if not args.no_extras:
+        also = {}
+        n = max(5, args.steps // 10)
+        # same shape, BSHD-contiguous memory viewed as BHSD (what a single-GPU Flux block hands over)
+        qb, kb, vb = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
+        _, ms = time_calls(lambda: ops.attn_fwd(qb, kb, vb), n, 3)
+        also["c2_flux1024_bshd_view"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        # ring of 4 KV chunks, merged in fp32 (the cast of the last fold is fused)
+        fn = usp._get_attention_function()
+        _, ms = time_calls(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), n, 3)
+        also["c3_flux_ring4"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        # the merge kernel alone: bytes per fold = 10*N*D + 12*N
+        N = B * H * S
+        acc = torch.randn(B, H, S, D, device=dev)
+        acc_l = torch.randn(B, H, S, device=dev)
+        blk_l = torch.randn(B, H, S, device=dev)
+        _, ms = time_calls(lambda: ops.lse_merge(acc, acc_l, q, blk_l), max(20, n), 5)
+        mbytes = 10.0 * N * D + 12.0 * N
+        also["lse_merge_fold"] = {"us": round(ms * 1e3, 2), "gbs": round(mbytes / ms / 1e6, 1),
+                                  "frac_hbm_peak": round(mbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": mbytes}
+        del acc, qb, kb, vb
+        # HunyuanVideo 720p one-GPU head shard
+        Bh, Hh, Sh = 1, 3, 118800 + 256
+        qh, kh, vh = make_inputs(Bh, Hh, Sh, D, 1004, dev)
+        _, ms = time_calls(lambda: ops.attn_fwd(qh, kh, vh), 5, 2)
+        fl = attn_flops(Bh, Hh, Sh, Sh, D)
+        also["c4_hunyuan720p_shard"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1),
+                                        "frac_bf16_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        del qh, kh, vh
+        # Wan2.1 720p head shard, fp8 e4m3fn + per-head scales -> bf16
+        Bw, Hw, Sw = 1, 5, 75600
+        qw, kw, vw = make_inputs(Bw, Hw, Sw, D, 1005, dev, rmsnorm=False)
+        (q8, qd), (k8, kd), (v8, vd) = (ops.fp8_quant(t) for t in (qw, kw, vw))
+        _, ms = time_calls(lambda: ops.attn_fwd(q8, k8, v8, q_descale=qd, k_descale=kd, v_descale=vd), 5, 2)
+        fl = attn_flops(Bw, Hw, Sw, Sw, D)
+        also["c5_wan720p_shard_fp8"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1),
+                                        "frac_fp8_peak": round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
+        _, ms = time_calls(lambda: ops.fp8_quant(qw), 10, 2)
+        also["fp8_quant_wan_shard"] = {"us": round(ms * 1e3, 1), "gbs": round(qw.numel() * 5.0 / ms / 1e6, 1)}
+        del qw, kw, vw, q8, k8, v8
+        result["also"] = also
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(q, k, v)
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
