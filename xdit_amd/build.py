@@ -28,9 +28,12 @@ def _hipcc():
     raise RuntimeError("hipcc not found")
 
 
+EXTRA_FLAGS = {}  # per-file additions
+
+
 def _compile(src):
     obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))

@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "common.h"
@@ -116,7 +117,13 @@ int xdit_attn_fwd(const xdit_attn_args* a) {
 
   hipError_t e;
   if ((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64)) {
-    e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, a->D, stream);
+    // 256 query rows per workgroup (8 wavefronts sharing each K/V tile: half the L2->LDS traffic)
+    // when that still yields enough workgroups to fill the 256 CUs, else 128 rows.
+    const int64_t big_tiles = (int64_t)a->B * a->H * ((a->Sq + 255) / 256);
+    static const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128" or "256": testing aid
+    int rows = (a->D == 128 && big_tiles >= 192) ? 256 : 128;
+    if (force != nullptr && a->D == 128) rows = std::atoi(force);
+    e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, a->D, rows, stream);
   } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
     if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
     e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, stream);

@@ -15,77 +15,25 @@
 // and the S^T accumulator registers are, after conversion to 16 bit, exactly the B operand of
 // the second product, so P never goes through LDS.
 //
-// LDS layout: a K (or V) tile is 64 rows of D 16-bit elements.  K is read with ds_read_b128
-// (lane -> one key row, 16 bytes), V with ds_read_b64_tr_b16 (16-lane group -> 4 key rows x 32
-// bytes).  A direct global->LDS load writes lane i at LDS offset base + 16*i, i.e. one 1 KiB
-// contiguous piece per wavefront instruction, so padding can only go BETWEEN those pieces.  Each
-// piece therefore holds rows {g, g+NG, g+2NG, ...} (NG pieces per tile) and pieces are
-// 1024 + PAD bytes apart: rows that are read together (consecutive rows) then sit in different
-// pieces, PAD bytes apart in bank space (PAD = 16 for the 16-byte K reads, 64 for the 64-byte V
-// reads), which makes both read patterns bank-conflict free while every read address is one
-// per-lane base plus a compile-time immediate.
-#include "common.h"
+// LDS layout: see attn_tiles.h.  The workgroup has NW = 4 or 8 wavefronts (128 or 256 query rows):
+// 8 wavefronts share every K/V tile, which halves the L2->LDS traffic per FLOP, and are used
+// when the problem still yields enough workgroups to fill the chip.
+#include "attn_tiles.h"
 #include "launchers.h"
 
 namespace xdit {
 
 constexpr int kRowsPerWave = 32;
-constexpr int kWaves = 4;
-constexpr int kRowsPerBlock = kRowsPerWave * kWaves;  // 128 query rows per workgroup
-constexpr int kKeysPerTile = 64;
-// A row maximum is replaced only when it grows by more than this many powers of two, so the
-// rescale of the output accumulator is skipped on almost every tile; exponentials stay <= 2^8.
-constexpr float kLazyRescaleLog2 = 8.0f;
+// K fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
+constexpr int kPrefetch = 4;
 
-template <typename T> struct Mfma16;
-template <> struct Mfma16<__bf16> {
-  typedef bf16x8 vec8;
-  typedef bf16x2 vec2;
-  static __device__ __forceinline__ f32x16 mma(vec8 a, vec8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-};
-template <> struct Mfma16<_Float16> {
-  typedef f16x8 vec8;
-  typedef f16x2 vec2;
-  static __device__ __forceinline__ f32x16 mma(vec8 a, vec8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-};
-
-// Tile geometry: ROWS_PER_PIECE rows fit one 1 KiB wavefront load, NG pieces per 64-key tile;
-// row r lives in piece r % NG at slot r / NG.
-template <int D> struct TileGeom {
-  static constexpr int ROW_BYTES = D * 2;
-  static constexpr int ROWS_PER_PIECE = 1024 / ROW_BYTES;
-  static constexpr int NG = kKeysPerTile / ROWS_PER_PIECE;
-  static constexpr int K_PITCH = 1024 + 16;
-  static constexpr int V_PITCH = 1024 + 64;
-  static constexpr int K_BYTES = NG * K_PITCH;
-  static constexpr int V_BYTES = NG * V_PITCH;
-  static constexpr int BUF_BYTES = K_BYTES + V_BYTES;
-};
-
-// Direct global->LDS load of 16 bytes per lane: lane i's data lands at LDS address lds + 16*i.
-// `base` (64-bit) and `lds` must be wavefront-uniform; `off` is the lane's byte offset from base.
-// Issued as inline assembly so that the compiler does not order later LDS reads of the OTHER
-// tile buffer behind it; completion is awaited explicitly with s_waitcnt vmcnt(0).
-__device__ __forceinline__ void load_lds_16(const void* base, unsigned off, unsigned lds) {
-  asm volatile(
-      "s_mov_b32 m0, %0\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %2"
-      :
-      : "s"(lds), "v"(off), "s"(base)
-      : "memory", "m0");
-}
-
-template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void attn_fwd_16_kernel(const AttnParams p) {
+template <typename T, int D, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(const AttnParams p) {
+  constexpr int kWaves = NW;
+  constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
   typedef typename Mfma16<T>::vec8 vec8;
   typedef typename Mfma16<T>::vec2 vec2;
   typedef TileGeom<D> G;
-  constexpr int LOADS = G::NG / kWaves;  // 1 KiB pieces per wavefront per tile (K and V each)
   constexpr int KSTEPS = D / 16;         // contraction steps of QK^T
   constexpr int DBLOCKS = D / 32;        // 32-row blocks of O^T
 
@@ -113,24 +61,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_16_kernel(const AttnParams p)
   for (int ks = 0; ks < KSTEPS; ks++) qf[ks] = *(const vec8*)(qptr + ks * 16);
 
   // ---- direct global->LDS tile loads ------------------------------------------------------
-  // Piece g = 4i + wave (i < LOADS) of a tile holds rows g, g+NG, g+2NG, ...; within the
-  // wavefront load lane -> (slot = lane / lanes-per-row, 16-byte column = lane % lanes-per-row).
-  // A load is "uniform 64-bit tile base + per-lane 32-bit byte offset"; the offsets of a full
-  // tile of segment 1 never change and live in registers.
+  // A tile is 2*NG pieces of 1 KiB (K pieces 0..NG-1, then V pieces): piece g of K (or V) holds
+  // rows g, g+NG, g+2NG, ...; wavefront w loads pieces w, w+NW, w+2NW, ...; within a piece
+  // lane -> (slot = lane / lanes-per-row, 16-byte column = lane % lanes-per-row).  A load is
+  // "uniform 64-bit tile base + per-lane 32-bit byte offset".
   const T* kbase1 = (const T*)p.k + b * p.ks_b + h * p.ks_h;
   const T* vbase1 = (const T*)p.v + b * p.vs_b + h * p.vs_h;
   const T* kbase2 = p.Sk2 > 0 ? (const T*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
   const T* vbase2 = p.Sk2 > 0 ? (const T*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
   constexpr int LANES_PER_ROW = G::ROW_BYTES / 16;
-  const int ld_slot = lane / LANES_PER_ROW;
-  const unsigned ld_colb = (lane % LANES_PER_ROW) * 16;  // byte offset inside the row
-  unsigned koffs[LOADS], voffs[LOADS];
-#pragma unroll
-  for (int i = 0; i < LOADS; i++) {
-    const unsigned r = 4 * i + wave + G::NG * ld_slot;
-    koffs[i] = r * (unsigned)(p.ks_s * 2) + ld_colb;
-    voffs[i] = r * (unsigned)(p.vs_s * 2) + ld_colb;
-  }
+  constexpr int PIECES = 2 * G::NG;
+  constexpr int LOADS = (PIECES + kWaves - 1) / kWaves;  // pieces per wavefront per tile
+  const int ld_row0 = G::NG * (lane / LANES_PER_ROW);       // row of this lane's slot within piece 0
+  const unsigned ld_colb = (lane % LANES_PER_ROW) * 16;     // byte offset inside the row
   const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS unsigned char*)smem;
 
   const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
@@ -140,39 +83,33 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_16_kernel(const AttnParams p)
   auto issue_tile = [&](int t, int buf) {
     const unsigned kdst = lds_base + buf * G::BUF_BYTES;
     const unsigned vdst = kdst + G::K_BYTES;
-    if (t < nt1 && (t + 1) * kKeysPerTile <= p.Sk) {  // full tile of segment 1
-      const T* kb = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
-      const T* vb = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
+    const T* kb;
+    const T* vb;
+    unsigned kss, vss;
+    int valid;
+    if (t < nt1) {
+      kb = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
+      vb = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
+      kss = (unsigned)(p.ks_s * 2); vss = (unsigned)(p.vs_s * 2);
+      valid = p.Sk - t * kKeysPerTile;
+    } else {
+      kb = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
+      vb = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
+      kss = (unsigned)(p.k2s_s * 2); vss = (unsigned)(p.v2s_s * 2);
+      valid = p.Sk2 - (t - nt1) * kKeysPerTile;
+    }
+    const int last = (valid < kKeysPerTile ? valid : kKeysPerTile) - 1;
 #pragma unroll
-      for (int i = 0; i < LOADS; i++) {
-        const int g = 4 * i + wave;
-        load_lds_16(kb, koffs[i], kdst + g * G::K_PITCH);
-        load_lds_16(vb, voffs[i], vdst + g * G::V_PITCH);
-      }
-    } else {  // partial tile and/or segment 2: recompute the offsets
-      const T* kb;
-      const T* vb;
-      unsigned kss, vss;
-      int valid;
-      if (t < nt1) {
-        kb = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
-        vb = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
-        kss = (unsigned)(p.ks_s * 2); vss = (unsigned)(p.vs_s * 2);
-        valid = p.Sk - t * kKeysPerTile;
-      } else {
-        kb = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
-        vb = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
-        kss = (unsigned)(p.k2s_s * 2); vss = (unsigned)(p.v2s_s * 2);
-        valid = p.Sk2 - (t - nt1) * kKeysPerTile;
-      }
-      const int last = (valid < kKeysPerTile ? valid : kKeysPerTile) - 1;
-#pragma unroll
-      for (int i = 0; i < LOADS; i++) {
-        const int g = 4 * i + wave;
-        int r = g + G::NG * ld_slot;
+    for (int i = 0; i < LOADS; i++) {
+      const int pi = wave + kWaves * i;  // wavefront-uniform
+      if (pi < PIECES) {
+        const bool is_v = pi >= G::NG;
+        const int g = is_v ? pi - G::NG : pi;
+        int r = g + ld_row0;
         r = r < last ? r : last;  // rows past the end of the segment re-read its last row
-        load_lds_16(kb, (unsigned)r * kss + ld_colb, kdst + g * G::K_PITCH);
-        load_lds_16(vb, (unsigned)r * vss + ld_colb, vdst + g * G::V_PITCH);
+        const unsigned off = __umul24((unsigned)r, is_v ? vss : kss) + ld_colb;
+        load_lds_16(is_v ? (const void*)vb : (const void*)kb, off,
+                    is_v ? vdst + g * G::V_PITCH : kdst + g * G::K_PITCH);
       }
     }
   };
@@ -321,32 +258,36 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_16_kernel(const AttnParams p)
   }
 }
 
-template <typename T, int D>
-static hipError_t launch_one(const AttnParams& q, dim3 grid, hipStream_t stream, bool& lds_ready) {
+template <typename T, int D, int NW>
+static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_ready) {
+  AttnParams q = p;
+  q.nq_tiles = (p.Sq + 32 * NW - 1) / (32 * NW);
+  q.total_tiles = p.B * p.H * q.nq_tiles;
+  q.tiles_per_xcd = (q.total_tiles + 7) / 8;
+  dim3 grid(q.tiles_per_xcd * 8);
   constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
   if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     lds_ready = true;
   }
-  hipLaunchKernelGGL((attn_fwd_16_kernel<T, D>), grid, dim3(256), lds, stream, q);
+  hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, NW>), grid, dim3(64 * NW), lds, stream, q);
   return hipGetLastError();
 }
 
 // Host-side launcher (called from the C ABI after argument validation).
-hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, hipStream_t stream) {
-  AttnParams q = p;
-  q.nq_tiles = (p.Sq + kRowsPerBlock - 1) / kRowsPerBlock;
-  q.total_tiles = p.B * p.H * q.nq_tiles;
-  q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  dim3 grid(q.tiles_per_xcd * 8);
-  static bool ready[4] = {false, false, false, false};
-  if (D == 128) {
-    return dtype_is_fp16 ? launch_one<_Float16, 128>(q, grid, stream, ready[0])
-                         : launch_one<__bf16, 128>(q, grid, stream, ready[1]);
+// rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12 wavefronts); the larger two are for
+// head_dim 128 only.
+hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream) {
+  static bool ready[8] = {false, false, false, false, false, false, false, false};
+  if (D == 128 && rows_per_block == 384) {
+    return dtype_is_fp16 ? launch_one<_Float16, 128, 12>(p, stream, ready[6]) : launch_one<__bf16, 128, 12>(p, stream, ready[7]);
+  } else if (D == 128 && rows_per_block == 256) {
+    return dtype_is_fp16 ? launch_one<_Float16, 128, 8>(p, stream, ready[4]) : launch_one<__bf16, 128, 8>(p, stream, ready[5]);
+  } else if (D == 128) {
+    return dtype_is_fp16 ? launch_one<_Float16, 128, 4>(p, stream, ready[0]) : launch_one<__bf16, 128, 4>(p, stream, ready[1]);
   } else if (D == 64) {
-    return dtype_is_fp16 ? launch_one<_Float16, 64>(q, grid, stream, ready[2])
-                         : launch_one<__bf16, 64>(q, grid, stream, ready[3]);
+    return dtype_is_fp16 ? launch_one<_Float16, 64, 4>(p, stream, ready[2]) : launch_one<__bf16, 64, 4>(p, stream, ready[3]);
   }
   return hipErrorInvalidValue;
 }
