@@ -31,6 +31,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+MEASURED_HBM_BYTES_PER_LAUNCH = 132.7e6  # Flux-1024 bf16 forward: 103.9 MB read + 28.75 MB written
 
 
 def make_inputs(B, H, S, D, seed, device, rmsnorm=True, dtype=torch.bfloat16):
@@ -155,7 +156,9 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by a 256 MiB
+            # copy in the same run (profiles/attn_fwd_bf16_flux1024_hbm_traffic.md)
+            "traffic": MEASURED_HBM_BYTES_PER_LAUNCH,
             "kernel": "attn_fwd_16_kernel<bf16,128>",
             "kernel_ms": round(ev_ms, 5),
         },
