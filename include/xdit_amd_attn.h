@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define XDIT_ATTN_ABI_VERSION 1
+#define XDIT_ATTN_ABI_VERSION 2
 
 typedef enum {
   XDIT_OK = 0,
@@ -89,10 +89,24 @@ typedef struct {
   const float* k_descale;
   const float* v_descale;
   int64_t descale_stride_b, descale_stride_h;
+  void* workspace;             /* optional scratch, 16-byte aligned; may be NULL (see below) */
+  int64_t workspace_bytes;
   void* stream;                /* hipStream_t; NULL = the null stream */
 } xdit_attn_args;
 
 int xdit_attn_fwd(const xdit_attn_args* args);
+
+/*
+ * Scratch bytes with which xdit_attn_fwd can balance this problem over the chip: when the number
+ * of query tiles is not a multiple of what the GPU holds at once, the key/value range of the
+ * tiles of the last, partly filled round is shared between workgroups, whose partial
+ * (out, lse) pairs go through the workspace and are folded by a second small kernel.
+ * Returns 0 when nothing would be gained, a negative xdit_status for invalid arguments
+ * (pointers are not inspected).  Passing no or too small a workspace to xdit_attn_fwd is always
+ * valid: the launch is then simply not balanced.  The workspace contents are undefined after the
+ * call and need no initialisation.  No counterpart in the reference (its kernels are vendor code).
+ */
+int64_t xdit_attn_workspace_bytes(const xdit_attn_args* args);
 
 /*
  * One fold of the ring online-softmax merge, in fp32:

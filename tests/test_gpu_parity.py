@@ -93,6 +93,37 @@ def test_two_kv_segments_equal_concatenation(gpu, dtype, Sk, Sk2):
     assert _err(o, ro) <= TOL[dtype][0] and _err(l, rl) <= TOL[dtype][1]
 
 
+@pytest.mark.parametrize("B,H,Sq,Sk,Sk2", [
+    (1, 1, 1280, 8192, 0),     # 10 query tiles on an empty chip: every tile's KV range is cut into many parts
+    (1, 3, 128, 6528, 0),      # 102 KV tiles, ranges of 4: a workgroup's range straddles two query tiles
+    (1, 2, 300, 4000, 100),    # partial last KV tile, second KV segment, partial last query tile
+    (2, 2, 200, 3333, 0),
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_balanced_launch_vs_oracle(gpu, dtype, B, H, Sq, Sk, Sk2):
+    """Problems whose query tiles do not fill the chip: the KV range of the tiles is shared between
+    workgroups and folded by the combine kernel.  Must match the oracle and the plain launch."""
+    g = torch.Generator().manual_seed(Sq + Sk)
+    q = torch.randn(B, H, Sq, 128, generator=g).to(dtype)
+    k, v = (torch.randn(B, H, Sk, 128, generator=g).to(dtype) for _ in range(2))
+    k2 = v2 = None
+    kk, vv = k, v
+    if Sk2:
+        k2, v2 = (torch.randn(B, H, Sk2, 128, generator=g).to(dtype) for _ in range(2))
+        kk, vv = torch.cat([k, k2], 2), torch.cat([v, v2], 2)
+    ro, rl = O.attn_fwd_ref(q, kk, vv)
+    dev = lambda t: None if t is None else t.to(gpu)
+    assert ops._lib.lib().xdit_attn_abi_version() >= 2
+    o, l = ops.attn_fwd(dev(q), dev(k), dev(v), k2=dev(k2), v2=dev(v2))
+    o1, l1 = ops.attn_fwd(dev(q), dev(k), dev(v), k2=dev(k2), v2=dev(v2), balance=False)
+    assert _err(o, ro) <= TOL[dtype][0] and _err(l, rl) <= TOL[dtype][1]
+    assert _err(o1, ro) <= TOL[dtype][0] and _err(l1, rl) <= TOL[dtype][1]
+    assert _err(o, o1.cpu()) <= 1e-2 and _err(l, l1.cpu()) <= 1e-5
+    # the workspace is scratch: a second call gives the same bits
+    o2, l2 = ops.attn_fwd(dev(q), dev(k), dev(v), k2=dev(k2), v2=dev(v2))
+    assert torch.equal(o, o2) and torch.equal(l, l2)
+
+
 # ---------------------------------------------------------------------------- named configurations
 def test_c1_pixart512_fp32_full(gpu):
     z = np.load(os.path.join(GOLD, "c1_pixart512.npz"))

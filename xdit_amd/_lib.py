@@ -9,7 +9,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libxdit_amd_attn.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 XDIT_OK = 0
 XDIT_ERR_INVALID_ARG = -1
@@ -58,6 +58,8 @@ class AttnArgs(ctypes.Structure):
         ("v_descale", ctypes.c_void_p),
         ("descale_stride_b", ctypes.c_int64),
         ("descale_stride_h", ctypes.c_int64),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_int64),
         ("stream", ctypes.c_void_p),
     ]
 
@@ -106,7 +108,7 @@ class QuantArgs(ctypes.Structure):
     ]
 
 
-EXPORTS = ("xdit_attn_fwd", "xdit_lse_merge", "xdit_fp8_quant", "xdit_attn_last_error", "xdit_attn_abi_version")
+EXPORTS = ("xdit_attn_fwd", "xdit_attn_workspace_bytes", "xdit_lse_merge", "xdit_fp8_quant", "xdit_attn_last_error", "xdit_attn_abi_version")
 
 _lib = None
 _lock = threading.Lock()
@@ -128,6 +130,8 @@ def lib():
         L = ctypes.CDLL(LIB_PATH)
         L.xdit_attn_fwd.argtypes = [ctypes.POINTER(AttnArgs)]
         L.xdit_attn_fwd.restype = ctypes.c_int
+        L.xdit_attn_workspace_bytes.argtypes = [ctypes.POINTER(AttnArgs)]
+        L.xdit_attn_workspace_bytes.restype = ctypes.c_int64
         L.xdit_lse_merge.argtypes = [ctypes.POINTER(MergeArgs)]
         L.xdit_lse_merge.restype = ctypes.c_int
         L.xdit_fp8_quant.argtypes = [ctypes.POINTER(QuantArgs)]

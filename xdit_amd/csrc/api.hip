@@ -52,6 +52,21 @@ int check_tensor(const char* name, const void* p, const xdit_strides& st, int es
   return 0;
 }
 
+// Query rows per workgroup for the 16-bit kernel: 384 (12 wavefronts sharing each K/V tile, 3 per
+// SIMD) or 256 (8) when that still yields enough workgroups to fill the 256 CUs, else 128.
+int rows_per_block_16(const xdit_attn_args* a) {
+  static const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128", "256" or "384": testing aid
+  if (a->D != 128) return 128;
+  if (force != nullptr) {
+    const int r = std::atoi(force);
+    if (r == 128 || r == 256 || r == 384) return r;
+  }
+  const int64_t bh = (int64_t)a->B * a->H;
+  if (bh * ((a->Sq + 383) / 384) >= 256) return 384;
+  if (bh * ((a->Sq + 255) / 256) >= 192) return 256;
+  return 128;
+}
+
 }  // namespace
 
 extern "C" {
@@ -113,17 +128,15 @@ int xdit_attn_fwd(const xdit_attn_args* a) {
   p.B = a->B; p.H = a->H;
   p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.scale = a->softmax_scale;
+  if (a->workspace != nullptr && a->workspace_bytes > 0 && aligned16(a->workspace)) {
+    p.ws_out = a->workspace;
+    p.ws_bytes = (size_t)a->workspace_bytes;
+  }
   hipStream_t stream = (hipStream_t)a->stream;
 
   hipError_t e;
   if ((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64)) {
-    // 256 query rows per workgroup (8 wavefronts sharing each K/V tile: half the L2->LDS traffic)
-    // when that still yields enough workgroups to fill the 256 CUs, else 128 rows.
-    const int64_t big_tiles = (int64_t)a->B * a->H * ((a->Sq + 255) / 256);
-    static const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128" or "256": testing aid
-    int rows = (a->D == 128 && big_tiles >= 192) ? 256 : 128;
-    if (force != nullptr && a->D == 128) rows = std::atoi(force);
-    e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, a->D, rows, stream);
+    e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, a->D, rows_per_block_16(a), stream);
   } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
     if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
     e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, stream);
@@ -133,6 +146,21 @@ int xdit_attn_fwd(const xdit_attn_args* a) {
   }
   if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
   return XDIT_OK;
+}
+
+int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
+  g_err[0] = 0;
+  if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
+  if (a->struct_size != sizeof(xdit_attn_args))
+    return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_attn_args));
+  if (a->B <= 0 || a->H <= 0 || a->Sq <= 0 || a->Sk <= 0 || a->Sk2 < 0 || a->Sq > (int64_t(1) << 30) ||
+      a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30))
+    return fail(XDIT_ERR_INVALID_ARG, "bad shape");
+  if (!((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64))) return 0;
+  xdit::AttnParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
+  return (int64_t)xdit::attn_fwd_16_workspace(p, a->D, rows_per_block_16(a));
 }
 
 int xdit_lse_merge(const xdit_merge_args* a) {

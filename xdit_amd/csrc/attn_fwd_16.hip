@@ -27,8 +27,14 @@ constexpr int kRowsPerWave = 32;
 // K fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
 constexpr int kPrefetch = 4;
 
+// One segment of work: the query tile `tile`, KV tiles [it0, it1).  With `part_out == nullptr` the
+// normalised result goes to the output tensors; otherwise the segment is one PART of a query tile
+// whose KV range is shared between workgroups, and its normalised partial output (in T) and
+// log-sum-exp go to the workspace slot (part_out, part_lse), [row][D] and [row], to be folded by
+// attn_combine_kernel.
 template <typename T, int D, int NW>
-__global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(const AttnParams p) {
+__device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char* smem, const int tile,
+                                             const int it0, const int it1, T* part_out, float* part_lse) {
   constexpr int kWaves = NW;
   constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
   typedef typename Mfma16<T>::vec8 vec8;
@@ -37,16 +43,12 @@ __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(
   constexpr int KSTEPS = D / 16;         // contraction steps of QK^T
   constexpr int DBLOCKS = D / 32;        // 32-row blocks of O^T
 
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // 2 x [K tile | V tile]
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int hh = lane >> 5;
 
-  const int tile = xcd_tile_index(blockIdx.x, p.tiles_per_xcd);
-  if (tile >= p.total_tiles) return;
   const int bh = tile / p.nq_tiles;
   const int qt = tile - bh * p.nq_tiles;
   const int b = bh / p.H;
@@ -140,20 +142,20 @@ __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
 
-  issue_tile(0, 0);
+  issue_tile(it0, 0);
   // Make the compiler account for the Q fragment loads here, before the loop: the tile loads
   // above are invisible to its outstanding-load bookkeeping, so any wait it placed for a Q
   // fragment inside the loop would also wait for the prefetch of the next tile.
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+v"(qf[ks]));
 
-  for (int t = 0; t < nt; t++) {
-    const int buf = t & 1;
+  for (int t = it0; t < it1; t++) {
+    const int buf = (t - it0) & 1;
     // Tile t has landed (this thread's loads) and, after the barrier, everyone's; the barrier
     // also means every wavefront is done reading the other buffer, which tile t+1 now overwrites.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (t + 1 < nt) issue_tile(t + 1, buf ^ 1);
+    if (t + 1 < it1) issue_tile(t + 1, buf ^ 1);
 
     const XDIT_LDS unsigned char* ktile =
         (const XDIT_LDS unsigned char*)(smem + buf * G::BUF_BYTES) + kbase_off;
@@ -239,8 +241,11 @@ __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(
   // ---- epilogue -----------------------------------------------------------------------------
   const float l_tot = sum_halves(l_part);
   const float inv = 1.0f / l_tot;
+  const float lse = (m_used * c + fast_log2(l_tot)) * kLn2;
   if (qrow < p.Sq) {
-    T* optr = (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
+    T* optr;
+    if (part_out != nullptr) optr = part_out + (wave * kRowsPerWave + l32) * D;
+    else optr = (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
 #pragma unroll
     for (int db = 0; db < DBLOCKS; db++)
 #pragma unroll
@@ -252,19 +257,149 @@ __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(
         vec4 ov = __builtin_convertvector(o, vec4);
         *(vec4*)(optr + 32 * db + 8 * a + 4 * hh) = ov;
       }
-    if (p.lse != nullptr && hh == 0) {
-      p.lse[b * p.ls_b + h * p.ls_h + qrow] = (m_used * c + fast_log2(l_tot)) * kLn2;
+    if (hh == 0) {
+      if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
+      else if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = lse;
     }
   }
+}
+
+// Workgroup -> work.  Plain launch: workgroup = one query tile over all KV tiles.  Balanced
+// launch (split_units > 0): the first split_full workgroups each take a whole query tile; the
+// KV iterations of the remaining query tiles, laid end to end, are cut into split_units equal
+// ranges of split_len iterations, one per workgroup, so that the last round of workgroups is as
+// full as the others.  A range may cover the end of one query tile and the start of the next.
+template <typename T, int D, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(const AttnParams p) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // 2 x [K tile | V tile]
+  constexpr int kRowsPerBlock = kRowsPerWave * NW;
+  const int nt = (p.Sk + kKeysPerTile - 1) / kKeysPerTile + (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  if (p.split_units == 0) {
+    const int tile = xcd_tile_index(blockIdx.x, p.tiles_per_xcd);
+    if (tile >= p.total_tiles) return;
+    attn_segment<T, D, NW>(p, smem, tile, 0, nt, nullptr, nullptr);
+    return;
+  }
+  const int w = blockIdx.x;
+  if (w < p.split_full) {
+    attn_segment<T, D, NW>(p, smem, xcd_tile_index(w, p.split_full >> 3), 0, nt, nullptr, nullptr);
+    return;
+  }
+  const int u = w - p.split_full;
+  const int rem_iters = (p.total_tiles - p.split_full) * nt;
+  int lin = u * p.split_len;
+  const int lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
+  bool first = true;
+  while (lin < lin_end) {
+    const int r = lin / nt;               // which of the remaining query tiles
+    const int it0 = lin - r * nt;
+    const int it1 = (lin_end - r * nt) < nt ? (lin_end - r * nt) : nt;
+    const int part = u - (r * nt) / p.split_len;  // ranges are consecutive: index within the tile
+    const int64_t slot = (int64_t)r * p.split_pmax + part;
+    if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
+    attn_segment<T, D, NW>(p, smem, p.split_full + r, it0, it1, (T*)p.ws_out + slot * kRowsPerBlock * D,
+                           p.ws_lse + slot * kRowsPerBlock);
+    first = false;
+    lin += it1 - it0;
+  }
+}
+
+// Folds the parts of every query tile that was split: out = sum_k exp(lse_k - L) out_k,
+// L = log sum_k exp(lse_k), in fp32; one thread per 8 head_dim elements of a row.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, const int rows_per_block, const int nt) {
+  constexpr int TPR = D / 8;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int rem_tiles = p.total_tiles - p.split_full;
+  const int64_t rrow = gid / TPR;  // row index within the remaining tiles
+  const int col = (int)(gid - rrow * TPR) * 8;
+  if (rrow >= (int64_t)rem_tiles * rows_per_block) return;
+  const int r = (int)(rrow / rows_per_block);
+  const int row = (int)(rrow - (int64_t)r * rows_per_block);
+  const int tile = p.split_full + r;
+  const int bh = tile / p.nq_tiles;
+  const int qt = tile - bh * p.nq_tiles;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+  const int qrow = qt * rows_per_block + row;
+  if (qrow >= p.Sq) return;
+  const int first_unit = (r * nt) / p.split_len;
+  const int last_unit = ((r + 1) * nt - 1) / p.split_len;
+  const int nparts = last_unit - first_unit + 1;
+  const float* lsep = p.ws_lse + ((int64_t)r * p.split_pmax) * rows_per_block + row;
+  float L = -INFINITY;
+  for (int k = 0; k < nparts; k++) L = fmaxf(L, lsep[(int64_t)k * rows_per_block]);
+  float denom = 0.f;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  typedef __attribute__((ext_vector_type(8))) T vec8;
+  for (int k = 0; k < nparts; k++) {
+    const float wk = __expf(lsep[(int64_t)k * rows_per_block] - L);
+    denom += wk;
+    const vec8 x = *(const vec8*)((const T*)p.ws_out + (((int64_t)r * p.split_pmax + k) * rows_per_block + row) * D + col);
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] += wk * (float)x[i];
+  }
+  const float inv = 1.0f / denom;
+  vec8 o;
+#pragma unroll
+  for (int i = 0; i < 8; i++) o[i] = (T)(acc[i] * inv);
+  *(vec8*)((T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s + col) = o;
+  if (col == 0 && p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = L + __logf(denom);
+}
+
+// Number of workgroups of NW wavefronts that are resident at once (LDS and wavefront slots).
+static int resident_workgroups(int NW) {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus = n;
+  }
+  return cus * (NW == 4 ? 2 : 1);
+}
+
+// Decide how to balance the launch; fills the split_* fields of q.  Returns the workspace bytes
+// the balanced launch needs (0 = plain launch).
+template <int D, int NW>
+static size_t plan_split(AttnParams& q) {
+  q.split_units = q.split_full = q.split_len = q.split_pmax = 0;
+  const int rows = 32 * NW;
+  const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  const int slots = resident_workgroups(NW);
+  const int T = q.total_tiles;
+  const int full = (T / slots) * slots;
+  const int rem = T - full;
+  if (rem == 0 || nt < 8) return 0;
+  int len = (int)(((int64_t)rem * nt + slots - 1) / slots);
+  if (len < 4) len = 4;
+  // Iterations of the critical path saved by filling the last round.  Idle CUs leave the busy
+  // ones more power (higher clock), so a partly filled round costs less than its length suggests;
+  // balance only when the saving clearly exceeds the cost of the extra prologues, the partial
+  // results and the combine pass (measured: about 10 iterations' worth).
+  if (nt - len < 48) return 0;
+  const int units = (int)(((int64_t)rem * nt + len - 1) / len);
+  q.split_full = full;
+  q.split_units = units;
+  q.split_len = len;
+  q.split_pmax = (nt + len - 1) / len + 1;
+  return (size_t)rem * q.split_pmax * rows * ((size_t)D * 2 + 4);
 }
 
 template <typename T, int D, int NW>
 static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_ready) {
   AttnParams q = p;
-  q.nq_tiles = (p.Sq + 32 * NW - 1) / (32 * NW);
+  constexpr int rows = 32 * NW;
+  q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  dim3 grid(q.tiles_per_xcd * 8);
+  const size_t need = plan_split<D, NW>(q);
+  if (need == 0 || p.ws_out == nullptr || p.ws_bytes < need) {
+    q.split_units = q.split_full = q.split_len = q.split_pmax = 0;
+  } else {
+    const int rem = q.total_tiles - q.split_full;
+    q.ws_lse = (float*)((unsigned char*)p.ws_out + (size_t)rem * q.split_pmax * rows * D * 2);
+  }
+  dim3 grid(q.split_units ? q.split_full + q.split_units : q.tiles_per_xcd * 8);
   constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
   if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
     hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -272,7 +407,30 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_
     lds_ready = true;
   }
   hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, NW>), grid, dim3(64 * NW), lds, stream, q);
+  if (q.split_units) {
+    const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+    const int64_t threads = (int64_t)(q.total_tiles - q.split_full) * rows * (D / 8);
+    hipLaunchKernelGGL((attn_combine_kernel<T, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, q, rows, nt);
+  }
   return hipGetLastError();
+}
+
+// Workspace bytes a balanced launch of this problem would use (0: none needed).
+template <int D, int NW>
+static size_t workspace_one(const AttnParams& p) {
+  AttnParams q = p;
+  constexpr int rows = 32 * NW;
+  q.nq_tiles = (p.Sq + rows - 1) / rows;
+  q.total_tiles = p.B * p.H * q.nq_tiles;
+  return plan_split<D, NW>(q);
+}
+
+size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block) {
+  if (D == 128 && rows_per_block == 384) return workspace_one<128, 12>(p);
+  if (D == 128 && rows_per_block == 256) return workspace_one<128, 8>(p);
+  if (D == 128) return workspace_one<128, 4>(p);
+  if (D == 64) return workspace_one<64, 4>(p);
+  return 0;
 }
 
 // Host-side launcher (called from the C ABI after argument validation).

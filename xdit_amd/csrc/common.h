@@ -50,6 +50,14 @@ struct AttnParams {
   int total_tiles;    // B * H * nq_tiles
   int tiles_per_xcd;  // ceil(total_tiles / 8)
   float scale;        // softmax scale
+  // balanced launch (see attn_fwd_16_kernel); all zero for a plain launch
+  int split_full;     // query tiles handled whole, by the first workgroups
+  int split_units;    // workgroups sharing the KV iterations of the remaining query tiles
+  int split_len;      // KV iterations per such workgroup
+  int split_pmax;     // workspace slots per remaining query tile
+  void* ws_out;       // workspace: partial outputs [tile][slot][row][D] in the output dtype ...
+  float* ws_lse;      // ... followed by partial log-sum-exps [tile][slot][row]
+  size_t ws_bytes;
 };
 
 // Combine a value across the two 32-lane halves of a wavefront (lane l with lane l^32).

@@ -44,13 +44,29 @@ def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+_WORKSPACE = {}
+
+
+def _workspace(device, nbytes):
+    """Per-device scratch tensor for balanced launches, grown on demand.  Calls on one stream are
+    ordered, so one buffer per (device, stream) can be reused from call to call."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    buf = _WORKSPACE.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+        _WORKSPACE[key] = buf
+    return buf
+
+
 def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
              q_descale=None, k_descale=None, v_descale=None, out_dtype=None, out=None,
-             return_lse=True):
+             return_lse=True, balance=True):
     """Non-causal attention forward on logical BHSD tensors -> (out BHSD, lse (B,H,Sq) fp32).
 
     `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
     with `k`/`v`.  For fp8 (torch.float8_e4m3fn) inputs the descales are (B, H) fp32 tensors.
+    `balance=False` withholds the scratch buffer with which the library evens out the last round
+    of workgroups (results then come from one workgroup per query tile).
     """
     if (k2 is None) != (v2 is None):
         raise ValueError("k2 and v2 should be None or not None simultaneously.")
@@ -115,6 +131,10 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
         a.descale_stride_b, a.descale_stride_h = d.stride(0), d.stride(1)
     a.stream = _stream(device)
     with torch.cuda.device(device):
+        need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) if balance else 0
+        if need > 0:
+            ws = _workspace(device, need)
+            a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
         _lib.check(_lib.lib().xdit_attn_fwd(ctypes.byref(a)))
     return out, lse
 
