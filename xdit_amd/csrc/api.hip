@@ -139,7 +139,7 @@ int xdit_attn_fwd(const xdit_attn_args* a) {
     e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, a->D, rows_per_block_16(a), stream);
   } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
     if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
-    e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, stream);
+    e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, rows_per_block_16(a), stream);
   } else {
     if (a->D > 128) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d above 128 is not implemented", a->D);
     e = xdit::launch_attn_fwd_f32(p, a->dtype, a->D, stream);
@@ -156,10 +156,11 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
   if (a->B <= 0 || a->H <= 0 || a->Sq <= 0 || a->Sk <= 0 || a->Sk2 < 0 || a->Sq > (int64_t(1) << 30) ||
       a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30))
     return fail(XDIT_ERR_INVALID_ARG, "bad shape");
-  if (!((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64))) return 0;
   xdit::AttnParams p;
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
+  if (a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128) return (int64_t)xdit::attn_fwd_fp8_workspace(p, rows_per_block_16(a));
+  if (!((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64))) return 0;
   return (int64_t)xdit::attn_fwd_16_workspace(p, a->D, rows_per_block_16(a));
 }
 

@@ -18,7 +18,7 @@
 // LDS layout: see attn_tiles.h.  The workgroup has NW = 4 or 8 wavefronts (128 or 256 query rows):
 // 8 wavefronts share every K/V tile, which halves the L2->LDS traffic per FLOP, and are used
 // when the problem still yields enough workgroups to fill the chip.
-#include "attn_tiles.h"
+#include "attn_split.h"
 #include "launchers.h"
 
 namespace xdit {
@@ -109,9 +109,8 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
         const int g = is_v ? pi - G::NG : pi;
         int r = g + ld_row0;
         r = r < last ? r : last;  // rows past the end of the segment re-read its last row
-        const unsigned off = __umul24((unsigned)r, is_v ? vss : kss) + ld_colb;
-        load_lds_16(is_v ? (const void*)vb : (const void*)kb, off,
-                    is_v ? vdst + g * G::V_PITCH : kdst + g * G::K_PITCH);
+        if (is_v) load_lds_16(vb, __umul24((unsigned)r, vss) + ld_colb, vdst + g * G::V_PITCH);
+        else load_lds_16(kb, __umul24((unsigned)r, kss) + ld_colb, kdst + g * G::K_PITCH);
       }
     }
   };
@@ -264,126 +263,17 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   }
 }
 
-// Workgroup -> work.  Plain launch: workgroup = one query tile over all KV tiles.  Balanced
-// launch (split_units > 0): the first split_full workgroups each take a whole query tile; the
-// KV iterations of the remaining query tiles, laid end to end, are cut into split_units equal
-// ranges of split_len iterations, one per workgroup, so that the last round of workgroups is as
-// full as the others.  A range may cover the end of one query tile and the start of the next.
 template <typename T, int D, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(const AttnParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // 2 x [K tile | V tile]
-  constexpr int kRowsPerBlock = kRowsPerWave * NW;
-  const int nt = (p.Sk + kKeysPerTile - 1) / kKeysPerTile + (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-  if (p.split_units == 0) {
-    const int tile = xcd_tile_index(blockIdx.x, p.tiles_per_xcd);
-    if (tile >= p.total_tiles) return;
-    attn_segment<T, D, NW>(p, smem, tile, 0, nt, nullptr, nullptr);
-    return;
-  }
-  const int w = blockIdx.x;
-  if (w < p.split_full) {
-    attn_segment<T, D, NW>(p, smem, xcd_tile_index(w, p.split_full >> 3), 0, nt, nullptr, nullptr);
-    return;
-  }
-  const int u = w - p.split_full;
-  const int rem_iters = (p.total_tiles - p.split_full) * nt;
-  int lin = u * p.split_len;
-  const int lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
-  bool first = true;
-  while (lin < lin_end) {
-    const int r = lin / nt;               // which of the remaining query tiles
-    const int it0 = lin - r * nt;
-    const int it1 = (lin_end - r * nt) < nt ? (lin_end - r * nt) : nt;
-    const int part = u - (r * nt) / p.split_len;  // ranges are consecutive: index within the tile
-    const int64_t slot = (int64_t)r * p.split_pmax + part;
-    if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
-    attn_segment<T, D, NW>(p, smem, p.split_full + r, it0, it1, (T*)p.ws_out + slot * kRowsPerBlock * D,
-                           p.ws_lse + slot * kRowsPerBlock);
-    first = false;
-    lin += it1 - it0;
-  }
+  run_workgroup<T, kRowsPerWave * NW, D>(p, [&](int tile, int it0, int it1, T* part_out, float* part_lse) {
+    attn_segment<T, D, NW>(p, smem, tile, it0, it1, part_out, part_lse);
+  });
 }
 
-// Folds the parts of every query tile that was split: out = sum_k exp(lse_k - L) out_k,
-// L = log sum_k exp(lse_k), in fp32; one thread per 8 head_dim elements of a row.
-template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, const int rows_per_block, const int nt) {
-  constexpr int TPR = D / 8;
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int rem_tiles = p.total_tiles - p.split_full;
-  const int64_t rrow = gid / TPR;  // row index within the remaining tiles
-  const int col = (int)(gid - rrow * TPR) * 8;
-  if (rrow >= (int64_t)rem_tiles * rows_per_block) return;
-  const int r = (int)(rrow / rows_per_block);
-  const int row = (int)(rrow - (int64_t)r * rows_per_block);
-  const int tile = p.split_full + r;
-  const int bh = tile / p.nq_tiles;
-  const int qt = tile - bh * p.nq_tiles;
-  const int b = bh / p.H;
-  const int h = bh - b * p.H;
-  const int qrow = qt * rows_per_block + row;
-  if (qrow >= p.Sq) return;
-  const int first_unit = (r * nt) / p.split_len;
-  const int last_unit = ((r + 1) * nt - 1) / p.split_len;
-  const int nparts = last_unit - first_unit + 1;
-  const float* lsep = p.ws_lse + ((int64_t)r * p.split_pmax) * rows_per_block + row;
-  float L = -INFINITY;
-  for (int k = 0; k < nparts; k++) L = fmaxf(L, lsep[(int64_t)k * rows_per_block]);
-  float denom = 0.f;
-  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  typedef __attribute__((ext_vector_type(8))) T vec8;
-  for (int k = 0; k < nparts; k++) {
-    const float wk = __expf(lsep[(int64_t)k * rows_per_block] - L);
-    denom += wk;
-    const vec8 x = *(const vec8*)((const T*)p.ws_out + (((int64_t)r * p.split_pmax + k) * rows_per_block + row) * D + col);
-#pragma unroll
-    for (int i = 0; i < 8; i++) acc[i] += wk * (float)x[i];
-  }
-  const float inv = 1.0f / denom;
-  vec8 o;
-#pragma unroll
-  for (int i = 0; i < 8; i++) o[i] = (T)(acc[i] * inv);
-  *(vec8*)((T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s + col) = o;
-  if (col == 0 && p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = L + __logf(denom);
-}
-
-// Number of workgroups of NW wavefronts that are resident at once (LDS and wavefront slots).
-static int resident_workgroups(int NW) {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cus = n;
-  }
-  return cus * (NW == 4 ? 2 : 1);
-}
-
-// Decide how to balance the launch; fills the split_* fields of q.  Returns the workspace bytes
-// the balanced launch needs (0 = plain launch).
-template <int D, int NW>
-static size_t plan_split(AttnParams& q) {
-  q.split_units = q.split_full = q.split_len = q.split_pmax = 0;
-  const int rows = 32 * NW;
-  const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-  const int slots = resident_workgroups(NW);
-  const int T = q.total_tiles;
-  const int full = (T / slots) * slots;
-  const int rem = T - full;
-  if (rem == 0 || nt < 8) return 0;
-  int len = (int)(((int64_t)rem * nt + slots - 1) / slots);
-  if (len < 4) len = 4;
-  // Iterations of the critical path saved by filling the last round.  Idle CUs leave the busy
-  // ones more power (higher clock), so a partly filled round costs less than its length suggests;
-  // balance only when the saving clearly exceeds the cost of the extra prologues, the partial
-  // results and the combine pass (measured: about 10 iterations' worth).
-  if (nt - len < 48) return 0;
-  const int units = (int)(((int64_t)rem * nt + len - 1) / len);
-  q.split_full = full;
-  q.split_units = units;
-  q.split_len = len;
-  q.split_pmax = (nt + len - 1) / len + 1;
-  return (size_t)rem * q.split_pmax * rows * ((size_t)D * 2 + 4);
-}
+// Workgroups of NW wavefronts resident at once: LDS and registers allow two 4-wavefront
+// workgroups per CU, one otherwise.
+static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 2 : 1); }
 
 template <typename T, int D, int NW>
 static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_ready) {
@@ -392,13 +282,7 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  const size_t need = plan_split<D, NW>(q);
-  if (need == 0 || p.ws_out == nullptr || p.ws_bytes < need) {
-    q.split_units = q.split_full = q.split_len = q.split_pmax = 0;
-  } else {
-    const int rem = q.total_tiles - q.split_full;
-    q.ws_lse = (float*)((unsigned char*)p.ws_out + (size_t)rem * q.split_pmax * rows * D * 2);
-  }
+  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2), rows, D, 2);
   dim3 grid(q.split_units ? q.split_full + q.split_units : q.tiles_per_xcd * 8);
   constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
   if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
@@ -422,7 +306,7 @@ static size_t workspace_one(const AttnParams& p) {
   constexpr int rows = 32 * NW;
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
-  return plan_split<D, NW>(q);
+  return plan_split(q, rows, resident_workgroups(NW), D, 2);
 }
 
 size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block) {

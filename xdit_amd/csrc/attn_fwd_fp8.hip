@@ -16,7 +16,7 @@
 // e4m3's normal range; the same factor is in the row sum, so it cancels in the output and is
 // subtracted from the log-sum-exp.  Logits are (q.k) * softmax_scale * q_descale * k_descale; the
 // output is multiplied by v_descale.
-#include "common.h"
+#include "attn_split.h"
 #include "launchers.h"
 
 namespace xdit {
@@ -24,9 +24,6 @@ namespace xdit {
 namespace fp8path {
 
 constexpr int kRowsPerWave = 32;
-constexpr int kWaves = 4;
-constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
-constexpr int kKeysPerTile = 64;
 constexpr int D = 128;
 constexpr float kPShift = 6.0f;           // P is scaled by 2^6 ...
 constexpr float kLazyRescaleLog2 = 2.0f;  // ... and the row max may lag by 2^2: P <= 2^8 < 448
@@ -41,22 +38,16 @@ constexpr int V_PITCH = 1024 + 32;
 constexpr int K_BYTES = NG * K_PITCH;
 constexpr int V_BYTES = NG * V_PITCH;
 constexpr int BUF_BYTES = K_BYTES + V_BYTES;
-constexpr int LOADS = NG / kWaves;  // 1 KiB pieces per wavefront per tile (K and V each)
+constexpr int PIECES = 2 * NG;  // 1 KiB pieces per tile: K pieces 0..NG-1, then V pieces
 
-__device__ __forceinline__ void load_lds_16(const void* base, unsigned off, unsigned lds) {
-  asm volatile(
-      "s_mov_b32 m0, %0\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %2"
-      :
-      : "s"(lds), "v"(off), "s"(base)
-      : "memory", "m0");
-}
-
-template <typename TO>
-__global__ __launch_bounds__(256, 2) void attn_fwd_fp8_kernel(const AttnParams p) {
+// One segment of work: query tile `tile`, KV tiles [it0, it1); see attn_split.h for part_out.
+template <typename TO, int NW>
+__device__ __forceinline__ void attn_segment_fp8(const AttnParams& p, unsigned char* smem, const int tile,
+                                                 const int it0, const int it1, TO* part_out, float* part_lse) {
   typedef unsigned char u8;
-  __shared__ __attribute__((aligned(1024))) u8 smem[2 * BUF_BYTES];
+  constexpr int kWaves = NW;
+  constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
+  constexpr int LOADS = (PIECES + kWaves - 1) / kWaves;  // pieces per wavefront per tile
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -64,8 +55,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_fp8_kernel(const AttnParams p
   const int l32 = lane & 31;
   const int hh = lane >> 5;
 
-  const int tile = xcd_tile_index(blockIdx.x, p.tiles_per_xcd);
-  if (tile >= p.total_tiles) return;
   const int bh = tile / p.nq_tiles;
   const int qt = tile - bh * p.nq_tiles;
   const int b = bh / p.H;
@@ -88,12 +77,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_fp8_kernel(const AttnParams p
   const u8* vbase1 = (const u8*)p.v + b * p.vs_b + h * p.vs_h;
   const u8* kbase2 = p.Sk2 > 0 ? (const u8*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
   const u8* vbase2 = p.Sk2 > 0 ? (const u8*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
-  const int ld_slot = lane >> 3;                // 8 lanes per 128-byte row
+  const int ld_row0 = NG * (lane >> 3);           // 8 lanes per 128-byte row: row of this lane's slot in piece 0
   const unsigned ld_colb = (lane & 7) * 16;
   const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS u8*)smem;
   const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
-  const int nt2 = (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-  const int nt = nt1 + nt2;
 
   auto issue_tile = [&](int t, int buf) {
     const unsigned kdst = lds_base + buf * BUF_BYTES;
@@ -116,11 +103,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_fp8_kernel(const AttnParams p
     const int last = (valid < kKeysPerTile ? valid : kKeysPerTile) - 1;
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
-      const int g = 4 * i + wave;
-      int r = g + NG * ld_slot;
-      r = r < last ? r : last;  // rows past the end of the segment re-read its last row
-      load_lds_16(kb, (unsigned)r * kss + ld_colb, kdst + g * K_PITCH);
-      load_lds_16(vb, (unsigned)r * vss + ld_colb, vdst + g * V_PITCH);
+      const int pi = wave + kWaves * i;  // wavefront-uniform
+      if (pi < PIECES) {
+        const bool is_v = pi >= NG;
+        const int g = is_v ? pi - NG : pi;
+        int r = g + ld_row0;
+        r = r < last ? r : last;  // rows past the end of the segment re-read its last row
+        if (is_v) load_lds_16(vb, __umul24((unsigned)r, vss) + ld_colb, vdst + g * V_PITCH);
+        else load_lds_16(kb, __umul24((unsigned)r, kss) + ld_colb, kdst + g * K_PITCH);
+      }
     }
   };
 
@@ -149,15 +140,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_fp8_kernel(const AttnParams p
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
 
-  issue_tile(0, 0);
+  issue_tile(it0, 0);
 #pragma unroll
   for (int ks = 0; ks < 2; ks++) asm volatile("" : "+v"(qf[ks]));
 
-  for (int t = 0; t < nt; t++) {
-    const int buf = t & 1;
+  for (int t = it0; t < it1; t++) {
+    const int buf = (t - it0) & 1;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (t + 1 < nt) issue_tile(t + 1, buf ^ 1);
+    if (t + 1 < it1) issue_tile(t + 1, buf ^ 1);
 
     const XDIT_LDS u8* ktile = (const XDIT_LDS u8*)(smem + buf * BUF_BYTES) + kbase_off;
     const XDIT_LDS u8* vtile = (const XDIT_LDS u8*)(smem + buf * BUF_BYTES + K_BYTES) + vbase_off;
@@ -240,8 +231,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_fp8_kernel(const AttnParams p
   // ---- epilogue -----------------------------------------------------------------------------
   const float l_tot = sum_halves(l_part);
   const float inv = sv / l_tot;
+  const float lse = (m_used * c - kPShift + fast_log2(l_tot)) * kLn2;
   if (qrow < p.Sq) {
-    TO* optr = (TO*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
+    TO* optr;
+    if (part_out != nullptr) optr = part_out + (wave * kRowsPerWave + l32) * D;
+    else optr = (TO*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
 #pragma unroll
     for (int db = 0; db < 4; db++)
 #pragma unroll
@@ -252,23 +246,66 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_fp8_kernel(const AttnParams p
         vec4 ov = __builtin_convertvector(o, vec4);
         *(vec4*)(optr + 32 * db + 8 * a + 4 * hh) = ov;
       }
-    if (p.lse != nullptr && hh == 0) {
-      p.lse[b * p.ls_b + h * p.ls_h + qrow] = (m_used * c - kPShift + fast_log2(l_tot)) * kLn2;
+    if (hh == 0) {
+      if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
+      else if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = lse;
     }
   }
 }
 
-}  // namespace fp8path
+template <typename TO, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 8 ? 2 : 3) void attn_fwd_fp8_kernel(const AttnParams p) {
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF_BYTES];
+  run_workgroup<TO, kRowsPerWave * NW, D>(p, [&](int tile, int it0, int it1, TO* part_out, float* part_lse) {
+    attn_segment_fp8<TO, NW>(p, smem, tile, it0, it1, part_out, part_lse);
+  });
+}
 
-hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, hipStream_t stream) {
+// Workgroups of NW wavefronts resident at once (3 wavefronts per SIMD by registers; 2 for NW = 8).
+static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 3 : 1); }
+
+template <typename TO, int NW>
+static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   AttnParams q = p;
-  q.nq_tiles = (p.Sq + fp8path::kRowsPerBlock - 1) / fp8path::kRowsPerBlock;
+  constexpr int rows = kRowsPerWave * NW;
+  q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  dim3 grid(q.tiles_per_xcd * 8);
-  if (out_is_fp16) hipLaunchKernelGGL((fp8path::attn_fwd_fp8_kernel<_Float16>), grid, dim3(256), 0, stream, q);
-  else hipLaunchKernelGGL((fp8path::attn_fwd_fp8_kernel<__bf16>), grid, dim3(256), 0, stream, q);
+  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2), rows, D, 2);
+  dim3 grid(q.split_units ? q.split_full + q.split_units : q.tiles_per_xcd * 8);
+  hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW>), grid, dim3(64 * NW), 0, stream, q);
+  if (q.split_units) {
+    const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+    const int64_t threads = (int64_t)(q.total_tiles - q.split_full) * rows * (D / 8);
+    hipLaunchKernelGGL((attn_combine_kernel<TO, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, q, rows, nt);
+  }
   return hipGetLastError();
+}
+
+template <int NW>
+static size_t workspace_one(const AttnParams& p) {
+  AttnParams q = p;
+  constexpr int rows = kRowsPerWave * NW;
+  q.nq_tiles = (p.Sq + rows - 1) / rows;
+  q.total_tiles = p.B * p.H * q.nq_tiles;
+  return plan_split(q, rows, resident_workgroups(NW), D, 2);
+}
+
+}  // namespace fp8path
+
+// rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12 wavefronts sharing each K/V tile).
+hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream) {
+  using namespace fp8path;
+  if (rows_per_block == 384) return out_is_fp16 ? launch_one<_Float16, 12>(p, stream) : launch_one<__bf16, 12>(p, stream);
+  if (rows_per_block == 256) return out_is_fp16 ? launch_one<_Float16, 8>(p, stream) : launch_one<__bf16, 8>(p, stream);
+  return out_is_fp16 ? launch_one<_Float16, 4>(p, stream) : launch_one<__bf16, 4>(p, stream);
+}
+
+size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block) {
+  using namespace fp8path;
+  if (rows_per_block == 384) return workspace_one<12>(p);
+  if (rows_per_block == 256) return workspace_one<8>(p);
+  return workspace_one<4>(p);
 }
 
 }  // namespace xdit

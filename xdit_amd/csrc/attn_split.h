@@ -1,0 +1,139 @@
+// Balanced launch shared by the attention kernels: when the query tiles do not fill a whole
+// number of rounds of resident workgroups, the KV iterations of the last round's tiles are cut
+// into equal ranges, one per workgroup; partial (out, lse) pairs go through a workspace and are
+// folded by attn_combine_kernel.
+#pragma once
+#include "attn_tiles.h"
+
+namespace xdit {
+
+// Workgroup -> segments of work.  `seg(tile, it0, it1, part_out, part_lse)` processes KV tiles
+// [it0, it1) of query tile `tile`; part_out == nullptr means "write the final result".
+// Plain launch (split_units == 0): workgroup = one query tile over all KV tiles.  Balanced launch:
+// the first split_full workgroups each take a whole query tile; the KV iterations of the
+// remaining query tiles, laid end to end, are cut into split_units ranges of split_len
+// iterations, one per workgroup.  A range may cover the end of one query tile and the start of
+// the next.  TO is the output element type, ROWS the query rows per workgroup.
+template <typename TO, int ROWS, int D, typename Seg>
+__device__ __forceinline__ void run_workgroup(const AttnParams& p, Seg seg) {
+  const int nt = (p.Sk + kKeysPerTile - 1) / kKeysPerTile + (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  if (p.split_units == 0) {
+    const int tile = xcd_tile_index(blockIdx.x, p.tiles_per_xcd);
+    if (tile >= p.total_tiles) return;
+    seg(tile, 0, nt, (TO*)nullptr, (float*)nullptr);
+    return;
+  }
+  const int w = blockIdx.x;
+  if (w < p.split_full) {
+    seg(xcd_tile_index(w, p.split_full >> 3), 0, nt, (TO*)nullptr, (float*)nullptr);
+    return;
+  }
+  const int u = w - p.split_full;
+  const int rem_iters = (p.total_tiles - p.split_full) * nt;
+  int lin = u * p.split_len;
+  const int lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
+  bool first = true;
+  while (lin < lin_end) {
+    const int r = lin / nt;               // which of the remaining query tiles
+    const int it0 = lin - r * nt;
+    const int it1 = (lin_end - r * nt) < nt ? (lin_end - r * nt) : nt;
+    const int part = u - (r * nt) / p.split_len;  // ranges are consecutive: index within the tile
+    const int64_t slot = (int64_t)r * p.split_pmax + part;
+    if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
+    seg(p.split_full + r, it0, it1, (TO*)p.ws_out + slot * ROWS * D, p.ws_lse + slot * ROWS);
+    first = false;
+    lin += it1 - it0;
+  }
+}
+
+// Folds the parts of every query tile that was split: out = sum_k exp(lse_k - L) out_k,
+// L = log sum_k exp(lse_k), in fp32; one thread per 8 head_dim elements of a row.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, const int rows_per_block, const int nt) {
+  constexpr int TPR = D / 8;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int rem_tiles = p.total_tiles - p.split_full;
+  const int64_t rrow = gid / TPR;  // row index within the remaining tiles
+  const int col = (int)(gid - rrow * TPR) * 8;
+  if (rrow >= (int64_t)rem_tiles * rows_per_block) return;
+  const int r = (int)(rrow / rows_per_block);
+  const int row = (int)(rrow - (int64_t)r * rows_per_block);
+  const int tile = p.split_full + r;
+  const int bh = tile / p.nq_tiles;
+  const int qt = tile - bh * p.nq_tiles;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+  const int qrow = qt * rows_per_block + row;
+  if (qrow >= p.Sq) return;
+  const int first_unit = (r * nt) / p.split_len;
+  const int last_unit = ((r + 1) * nt - 1) / p.split_len;
+  const int nparts = last_unit - first_unit + 1;
+  const float* lsep = p.ws_lse + ((int64_t)r * p.split_pmax) * rows_per_block + row;
+  float L = -INFINITY;
+  for (int k = 0; k < nparts; k++) L = fmaxf(L, lsep[(int64_t)k * rows_per_block]);
+  float denom = 0.f;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  typedef __attribute__((ext_vector_type(8))) T vec8;
+  for (int k = 0; k < nparts; k++) {
+    const float wk = __expf(lsep[(int64_t)k * rows_per_block] - L);
+    denom += wk;
+    const vec8 x = *(const vec8*)((const T*)p.ws_out + (((int64_t)r * p.split_pmax + k) * rows_per_block + row) * D + col);
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] += wk * (float)x[i];
+  }
+  const float inv = 1.0f / denom;
+  vec8 o;
+#pragma unroll
+  for (int i = 0; i < 8; i++) o[i] = (T)(acc[i] * inv);
+  *(vec8*)((T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s + col) = o;
+  if (col == 0 && p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = L + __logf(denom);
+}
+
+// Compute units of the current device (cached).
+static inline int resident_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus = n;
+  }
+  return cus;
+}
+
+// Decide how to balance the launch; fills the split_* fields of q.  Returns the workspace bytes
+// the balanced launch needs (0 = plain launch).
+// `rows` query rows per workgroup, `slots` workgroups resident at once, `out_bytes` per output element.
+static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int out_bytes) {
+  q.split_units = q.split_full = q.split_len = q.split_pmax = 0;
+  const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  const int T = q.total_tiles;
+  const int full = (T / slots) * slots;
+  const int rem = T - full;
+  if (rem == 0 || nt < 8) return 0;
+  int len = (int)(((int64_t)rem * nt + slots - 1) / slots);
+  if (len < 4) len = 4;
+  // Iterations of the critical path saved by filling the last round.  Idle CUs leave the busy
+  // ones more power (higher clock), so a partly filled round costs less than its length suggests;
+  // balance only when the saving clearly exceeds the cost of the extra prologues, the partial
+  // results and the combine pass (measured: about 10 iterations' worth).
+  if (nt - len < 48) return 0;
+  const int units = (int)(((int64_t)rem * nt + len - 1) / len);
+  q.split_full = full;
+  q.split_units = units;
+  q.split_len = len;
+  q.split_pmax = (nt + len - 1) / len + 1;
+  return (size_t)rem * q.split_pmax * rows * ((size_t)D * out_bytes + 4);
+}
+
+// Point ws_lse behind the partial outputs, or fall back to a plain launch when the caller gave no
+// (or too small a) workspace.
+static inline void bind_workspace(AttnParams& q, const AttnParams& p, size_t need, int rows, int D, int out_bytes) {
+  if (need == 0 || p.ws_out == nullptr || p.ws_bytes < need) {
+    q.split_units = q.split_full = q.split_len = q.split_pmax = 0;
+  } else {
+    const int rem = q.total_tiles - q.split_full;
+    q.ws_lse = (float*)((unsigned char*)p.ws_out + (size_t)rem * q.split_pmax * rows * D * out_bytes);
+  }
+}
+
+}  // namespace xdit
