@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-MEASURED_HBM_BYTES_PER_LAUNCH = 132.7e6  # Flux-1024 bf16 forward: 103.9 MB read + 28.75 MB written
+MEASURED_HBM_BYTES_PER_LAUNCH = 213.3e6  # Flux-1024 bf16 step: 152.7 MB read + 60.6 MB written (attention + combine kernels)
 
 
 def make_inputs(B, H, S, D, seed, device, rmsnorm=True, dtype=torch.bfloat16):
@@ -156,10 +156,10 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-            # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by a 256 MiB
-            # copy in the same run (profiles/attn_fwd_bf16_flux1024_hbm_traffic.md)
+            # HBM bytes per step from rocprofv3 FETCH_SIZE / WRITE_SIZE counters, each scaled by the
+            # same counter's reading for a 256 MiB copy in the same run (--copy-calibration)
             "traffic": MEASURED_HBM_BYTES_PER_LAUNCH,
-            "kernel": "attn_fwd_16_kernel<bf16,128>",
+            "kernel": "attn_fwd_16_kernel<bf16,128,12> (+ attn_combine_kernel<bf16,128> for the shared last round)",
             "kernel_ms": round(ev_ms, 5),
         },
     }
@@ -167,6 +167,9 @@ def main():
     if not args.no_extras:
         also = {}
         n = max(5, args.steps // 10)
+        # the plain launch (one workgroup per query tile, no shared last round, no combine kernel)
+        _, ms = time_calls(lambda: ops.attn_fwd(q, k, v, out=out, balance=False), n, 3)
+        also["c2_flux1024_plain_launch"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
         # same shape, BSHD-contiguous memory viewed as BHSD (what a single-GPU Flux block hands over)
         qb, kb, vb = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
         _, ms = time_calls(lambda: ops.attn_fwd(qb, kb, vb), n, 3)

@@ -124,6 +124,61 @@ def test_balanced_launch_vs_oracle(gpu, dtype, B, H, Sq, Sk, Sk2):
     assert torch.equal(o, o2) and torch.equal(l, l2)
 
 
+@pytest.fixture
+def force_rows(monkeypatch):
+    """Pins the query rows per workgroup (128 / 256 / 384: 4 / 8 / 12 wavefronts) that the library
+    would otherwise pick from the problem size; the library reads the variable on every call."""
+    def set_rows(rows):
+        monkeypatch.setenv("XDIT_ATTN_ROWS", str(rows))
+    return set_rows
+
+
+@pytest.mark.parametrize("rows", [128, 256, 384])
+@pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8"])
+@pytest.mark.parametrize("B,H,Sq,Sk,Sk2", [
+    (1, 2, 1000, 777, 0),       # several workgroups per head, partial last query tile and KV tile
+    (1, 1, 385, 8192, 0),       # balanced launch: KV ranges shared between workgroups
+    (1, 3, 700, 5000, 90),      # balanced launch with a second KV segment
+    (2, 2, 50, 64, 1),          # fewer query rows than one workgroup covers
+])
+def test_workgroup_shapes_vs_oracle(gpu, force_rows, rows, kind, B, H, Sq, Sk, Sk2):
+    """Every workgroup shape of the 16-bit and fp8 kernels, with and without the balanced launch,
+    against the oracle on the same inputs."""
+    force_rows(rows)
+    g = torch.Generator().manual_seed(rows + Sq + Sk)
+    mk = lambda n: torch.randn(B, H, n, 128, generator=g)
+    q, k, v = mk(Sq), mk(Sk), mk(Sk)
+    k2, v2 = (mk(Sk2), mk(Sk2)) if Sk2 else (None, None)
+    dev = lambda t: None if t is None else t.to(gpu)
+    if kind == "fp8":
+        kall = k if k2 is None else torch.cat([k, k2], 2)
+        vall = v if v2 is None else torch.cat([v, v2], 2)
+        (q8, qd), (k8, kd), (v8, vd) = (O.per_head_quant_ref(t) for t in (q, kall, vall))
+        ro, rl = O.attn_fwd_ref(O.dequant(q8, qd), O.dequant(k8, kd), O.dequant(v8, vd))
+        kw = dict(q_descale=dev(qd), k_descale=dev(kd), v_descale=dev(vd))
+        if Sk2:
+            kw.update(k2=dev(k8[:, :, Sk:].contiguous()), v2=dev(v8[:, :, Sk:].contiguous()))
+            k8, v8 = k8[:, :, :Sk].contiguous(), v8[:, :, :Sk].contiguous()
+        args = (dev(q8), dev(k8), dev(v8))
+        tol_o, tol_l = 6e-2, 1e-3
+    else:
+        dt = torch.bfloat16 if kind == "bf16" else torch.float16
+        q, k, v = q.to(dt), k.to(dt), v.to(dt)
+        kall, vall = k, v
+        kw = {}
+        if Sk2:
+            k2, v2 = k2.to(dt), v2.to(dt)
+            kall, vall = torch.cat([k, k2], 2), torch.cat([v, v2], 2)
+            kw.update(k2=dev(k2), v2=dev(v2))
+        ro, rl = O.attn_fwd_ref(q, kall, vall)
+        args = (dev(q), dev(k), dev(v))
+        tol_o, tol_l = TOL[dt]
+    o, l = ops.attn_fwd(*args, **kw)
+    o1, l1 = ops.attn_fwd(*args, balance=False, **kw)
+    assert _err(o, ro) <= tol_o and _err(l, rl) <= tol_l
+    assert _err(o1, ro) <= tol_o and _err(l1, rl) <= tol_l
+
+
 # ---------------------------------------------------------------------------- named configurations
 def test_c1_pixart512_fp32_full(gpu):
     z = np.load(os.path.join(GOLD, "c1_pixart512.npz"))

@@ -55,8 +55,8 @@ int check_tensor(const char* name, const void* p, const xdit_strides& st, int es
 // Query rows per workgroup for the 16-bit kernel: 384 (12 wavefronts sharing each K/V tile, 3 per
 // SIMD) or 256 (8) when that still yields enough workgroups to fill the 256 CUs, else 128.
 int rows_per_block_16(const xdit_attn_args* a) {
-  static const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128", "256" or "384": testing aid
   if (a->D != 128) return 128;
+  const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128", "256" or "384": testing aid, read per call
   if (force != nullptr) {
     const int r = std::atoi(force);
     if (r == 128 || r == 256 || r == 384) return r;

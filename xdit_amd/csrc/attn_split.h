@@ -74,12 +74,22 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, c
   float denom = 0.f;
   float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   typedef __attribute__((ext_vector_type(8))) T vec8;
-  for (int k = 0; k < nparts; k++) {
-    const float wk = __expf(lsep[(int64_t)k * rows_per_block] - L);
-    denom += wk;
-    const vec8 x = *(const vec8*)((const T*)p.ws_out + (((int64_t)r * p.split_pmax + k) * rows_per_block + row) * D + col);
+  const T* part0 = (const T*)p.ws_out + (((int64_t)r * p.split_pmax) * rows_per_block + row) * D + col;
+  for (int k0 = 0; k0 < nparts; k0 += 4) {  // four parts in flight per thread
+    vec8 x[4];
+    float w[4];
 #pragma unroll
-    for (int i = 0; i < 8; i++) acc[i] += wk * (float)x[i];
+    for (int j = 0; j < 4; j++) {
+      const int k = k0 + j < nparts ? k0 + j : nparts - 1;
+      x[j] = *(const vec8*)(part0 + (int64_t)k * rows_per_block * D);
+      w[j] = k0 + j < nparts ? __expf(lsep[(int64_t)k * rows_per_block] - L) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      denom += w[j];
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[i] += w[j] * (float)x[j][i];
+    }
   }
   const float inv = 1.0f / denom;
   vec8 o;
