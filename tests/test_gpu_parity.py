@@ -422,3 +422,37 @@ def test_runs_on_the_callers_stream(gpu):
         o, l = ops.attn_fwd(q2, k, v)
     s.synchronize()
     assert torch.equal(o, ref_o) and torch.equal(l, ref_l)
+
+
+# ---------------------------------------------------------------------------- torch.library ops
+def test_custom_ops_opcheck_and_compile(gpu):
+    """The registered ops pass torch's own consistency checks (schema, fake vs real outputs,
+    functionalisation of the in-place merge) and a compiled caller gives the eager bits without a
+    graph break."""
+    from xdit_amd import custom_ops  # noqa: F401
+    q, k, v = O.make_qkv(1, 2, 300, 128, seed=61, dtype=torch.bfloat16)
+    jk, jv = (t[:, :, :40].contiguous() for t in O.make_qkv(1, 2, 64, 128, seed=62, dtype=torch.bfloat16)[1:])
+    q, k, v, jk, jv = (t.to(gpu) for t in (q, k, v, jk, jv))
+    tests = ("test_schema", "test_faketensor", "test_autograd_registration")
+    torch.library.opcheck(torch.ops.xdit_amd.attn_fwd.default, (q, k, v, 128 ** -0.5), test_utils=tests)
+    torch.library.opcheck(torch.ops.xdit_amd.attn_fwd_joint.default, (q, k, v, jk, jv, 128 ** -0.5), test_utils=tests)
+    torch.library.opcheck(torch.ops.xdit_amd.fp8_quant.default, (q, True), test_utils=tests)
+    o, l = ops.attn_fwd(q, k, v)
+    acc_o, acc_l = o.float(), l.clone()
+    torch.library.opcheck(torch.ops.xdit_amd.lse_merge.default, (acc_o, acc_l, o, l, False), test_utils=tests)
+
+    eager = AB._mi355_attn_call(q, k, v, 0.0, False, joint_kv=(jk, jv, "rear"))
+
+    def block(q, k, v, jk, jv):
+        out, lse = AB._mi355_attn_call(q * 1, k, v, 0.0, False, joint_kv=(jk, jv, "rear"))
+        return out + 0, lse
+
+    co, cl = torch.compile(block, backend="aot_eager", fullgraph=True)(q, k, v, jk, jv)
+    assert torch.equal(co, eager[0]) and torch.equal(cl, eager[1])
+
+    def fp8_block(q, k, v):
+        return AB._mi355_fp8_attn_call(q, k, v, 0.0, False)
+
+    e8 = fp8_block(q, k, v)
+    c8 = torch.compile(fp8_block, backend="aot_eager", fullgraph=True)(q, k, v)
+    assert torch.equal(c8[0], e8[0]) and torch.equal(c8[1], e8[1])

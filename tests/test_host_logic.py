@@ -117,3 +117,72 @@ def test_legacy_ring_argument_errors():
         layer(None, q, q, q, joint_tensor_query=q)
     with pytest.raises(NotImplementedError):
         ring.update_out_and_lse(None, None, q, torch.zeros(1, 2, 8), slice_=(slice(0, 1),))
+
+
+def test_custom_ops_fake_implementations_describe_the_outputs():
+    """The `torch.library` ops (pattern of attention_backend.py:383-399 in the reference) must
+    trace on meta tensors: shapes, dtypes and contiguity of what the kernels return."""
+    from xdit_amd import custom_ops  # noqa: F401
+    B, H, Sq, Sk, D = 2, 3, 40, 70, 128
+    # BSHD memory viewed as BHSD, as a Flux block hands it over
+    q = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="meta").transpose(1, 2)
+    k = torch.empty(B, Sk, H, D, dtype=torch.bfloat16, device="meta").transpose(1, 2)
+    out, lse = torch.ops.xdit_amd.attn_fwd(q, k, k, 0.1)
+    assert out.shape == (B, H, Sq, D) and out.dtype == torch.bfloat16 and out.is_contiguous()
+    assert lse.shape == (B, H, Sq) and lse.dtype == torch.float32
+    k2 = torch.empty(B, H, 9, D, dtype=torch.bfloat16, device="meta")
+    out, lse = torch.ops.xdit_amd.attn_fwd_joint(q, k, k, k2, k2, 0.1)
+    assert out.shape == (B, H, Sq, D) and lse.shape == (B, H, Sq)
+    q8 = torch.empty(B, H, Sq, D, dtype=torch.float8_e4m3fn, device="meta")
+    k8 = torch.empty(B, H, Sk, D, dtype=torch.float8_e4m3fn, device="meta")
+    d = torch.empty(B, H, device="meta")
+    out, lse = torch.ops.xdit_amd.attn_fwd_fp8(q8, k8, k8, d, d, d, 0.1, True)
+    assert out.dtype == torch.float16 and out.shape == (B, H, Sq, D) and lse.dtype == torch.float32
+    out, _ = torch.ops.xdit_amd.attn_fwd_fp8(q8, k8, k8, d, d, d, 0.1, False)
+    assert out.dtype == torch.bfloat16
+    y, ds = torch.ops.xdit_amd.fp8_quant(q, False)
+    assert y.dtype == torch.float8_e4m3fn and y.shape == q.shape and y.is_contiguous() and ds.shape == (B, H)
+    # there is no CPU implementation behind the ops either
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.xdit_amd.attn_fwd(torch.zeros(1, 1, 4, 128), torch.zeros(1, 1, 4, 128), torch.zeros(1, 1, 4, 128), 0.1)
+
+
+def test_plugin_install_takes_over_registry_members_by_name():
+    """`plugin.install` against a stand-in for xfuser.core.distributed.attention_backend (an enum
+    plus a dict registry, attention_backend.py:23, :429-463)."""
+    import types
+    from enum import Enum
+    from xdit_amd import plugin
+
+    class AttentionBackendType(Enum):
+        SDPA = "SDPA"
+        AITER = "AITER"
+        AITER_FP8 = "AITER FP8"
+
+    old = lambda *a, **k: "old"
+    mod = types.SimpleNamespace(AttentionBackendType=AttentionBackendType,
+                                ATTENTION_FUNCTION_REGISTRY={AttentionBackendType.AITER: old})
+    replaced = plugin.install(mod)
+    reg = mod.ATTENTION_FUNCTION_REGISTRY
+    assert reg[AttentionBackendType.AITER].__name__ == "_mi355_attn_call"
+    assert reg[AttentionBackendType.AITER_FP8].__name__ == "_mi355_fp8_attn_call"
+    # the installed functions have the registry prototype and the same argument domain
+    q = torch.zeros(1, 2, 4, 128, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        reg[AttentionBackendType.AITER](q, q, q, 0.0, True)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        reg[AttentionBackendType.AITER](q, q, q, 0.0, False)
+    plugin.uninstall(replaced, mod)
+    assert reg[AttentionBackendType.AITER] is old and AttentionBackendType.AITER_FP8 not in reg
+    with pytest.raises(ValueError):
+        plugin.install(mod, names={"nope": old})
+
+
+def test_default_backend_by_name():
+    usp.set_default_backend("mi355_fp8")
+    try:
+        assert usp._DEFAULT_BACKEND is AB.AttentionBackendType.MI355_FP8
+        with pytest.raises(ValueError):
+            usp.set_default_backend("flash_9")
+    finally:
+        usp.set_default_backend(AB.AttentionBackendType.MI355)

@@ -11,6 +11,7 @@ from enum import Enum
 
 import torch
 
+from . import custom_ops  # noqa: F401  (registers torch.ops.xdit_amd.*)
 from . import ops
 
 ATTENTION_FUNCTION_REGISTRY = {}
@@ -66,7 +67,14 @@ def _mi355_attn_call(query, key, value, dropout_p, is_causal, attention_kwargs=N
     (attention_backend.py:790).  Returns (out BHSD in query's dtype, lse (B,H,S) fp32)."""
     _check_call(dropout_p, is_causal, attention_kwargs)
     k1, v1, k2, v2 = _split_joint(key, value, joint_kv)
-    return ops.attn_fwd(query, k1, v1, softmax_scale=query.shape[-1] ** -0.5, k2=k2, v2=v2)
+    scale = query.shape[-1] ** -0.5
+    if torch.compiler.is_compiling():
+        # under torch.compile the call goes through the registered custom ops (fake
+        # implementations describe the outputs, so tracing does not break the graph)
+        if k2 is None:
+            return torch.ops.xdit_amd.attn_fwd(query, k1, v1, scale)
+        return torch.ops.xdit_amd.attn_fwd_joint(query, k1, v1, k2, v2, scale)
+    return ops.attn_fwd(query, k1, v1, softmax_scale=scale, k2=k2, v2=v2)
 
 
 def get_dtype_max(dtype):
@@ -83,7 +91,10 @@ def per_tensor_quant(x, scale=None, scale_dtype=torch.float32, quant_dtype=torch
     if quant_dtype != torch.float8_e4m3fn:
         raise NotImplementedError("only float8_e4m3fn (the fp8 format of gfx950) is supported")
     if scale is None and dtypeMax in (None, get_dtype_max(quant_dtype)):
-        y, descale = ops.fp8_quant(x, per_tensor=True)
+        if torch.compiler.is_compiling():
+            y, descale = torch.ops.xdit_amd.fp8_quant(x, True)
+        else:
+            y, descale = ops.fp8_quant(x, per_tensor=True)
         return y, descale.to(scale_dtype)
     if scale is None:
         scale = torch.abs(x.to(torch.float32)).max() / dtypeMax
@@ -113,4 +124,6 @@ def _mi355_fp8_attn_call(query, key, value, dropout_p, is_causal, attention_kwar
     q8, qd = per_tensor_quant(query)
     k8, kd = per_tensor_quant(key)
     v8, vd = per_tensor_quant(value)
+    if torch.compiler.is_compiling():
+        return torch.ops.xdit_amd.attn_fwd_fp8(q8, k8, v8, qd, kd, vd, scale, out_dtype == torch.float16)
     return ops.attn_fwd(q8, k8, v8, softmax_scale=scale, q_descale=qd, k_descale=kd, v_descale=vd, out_dtype=out_dtype)

@@ -1,0 +1,98 @@
+"""`torch.library` custom ops over the HIP entry points, so `torch.compile` can trace through them.
+
+The reference wraps a vendor kernel the same way (xfuser/core/distributed/attention_backend.py:383-399:
+`@custom_op("xfuser::flydsl_attn_kernel", mutates_args=())` plus a `register_fake` that returns
+`torch.empty_like(query)`).  Here every op has a device implementation that calls the C ABI
+(`xdit_amd.ops`) and a fake implementation that only describes the outputs:
+
+    xdit_amd::attn_fwd        (q, k, v, softmax_scale)                      -> (out, lse)
+    xdit_amd::attn_fwd_joint  (q, k, v, k2, v2, softmax_scale)              -> (out, lse)
+    xdit_amd::attn_fwd_fp8    (q, k, v, q_descale, k_descale, v_descale,
+                               softmax_scale, out_fp16)                     -> (out, lse)
+    xdit_amd::lse_merge       (acc_out, acc_lse, block_out, block_lse, first)   in place
+    xdit_amd::lse_merge_final (acc_out, acc_lse, block_out, block_lse, final_out)  in place
+    xdit_amd::fp8_quant       (x, per_tensor)                               -> (y, descale)
+
+All tensors are logical BHSD (any B/H/S strides); outputs are BHSD-contiguous, lse is (B,H,Sq)
+fp32.  The ops are registered for GPU tensors only: there is no CPU implementation.
+"""
+from typing import Tuple
+
+import torch
+from torch.library import custom_op, register_fake
+
+from . import ops
+
+Tensor = torch.Tensor
+
+
+def _fake_out_lse(query: Tensor, out_dtype) -> Tuple[Tensor, Tensor]:
+    B, H, Sq, D = query.shape
+    return (query.new_empty((B, H, Sq, D), dtype=out_dtype),
+            query.new_empty((B, H, Sq), dtype=torch.float32))
+
+
+@custom_op("xdit_amd::attn_fwd", mutates_args=(), device_types="cuda")
+def attn_fwd(query: Tensor, key: Tensor, value: Tensor, softmax_scale: float) -> Tuple[Tensor, Tensor]:
+    return ops.attn_fwd(query, key, value, softmax_scale=softmax_scale)
+
+
+@register_fake("xdit_amd::attn_fwd")
+def _attn_fwd_fake(query, key, value, softmax_scale):
+    return _fake_out_lse(query, query.dtype)
+
+
+@custom_op("xdit_amd::attn_fwd_joint", mutates_args=(), device_types="cuda")
+def attn_fwd_joint(query: Tensor, key: Tensor, value: Tensor, key2: Tensor, value2: Tensor,
+                   softmax_scale: float) -> Tuple[Tensor, Tensor]:
+    return ops.attn_fwd(query, key, value, softmax_scale=softmax_scale, k2=key2, v2=value2)
+
+
+@register_fake("xdit_amd::attn_fwd_joint")
+def _attn_fwd_joint_fake(query, key, value, key2, value2, softmax_scale):
+    return _fake_out_lse(query, query.dtype)
+
+
+@custom_op("xdit_amd::attn_fwd_fp8", mutates_args=(), device_types="cuda")
+def attn_fwd_fp8(query: Tensor, key: Tensor, value: Tensor, q_descale: Tensor, k_descale: Tensor,
+                 v_descale: Tensor, softmax_scale: float, out_fp16: bool) -> Tuple[Tensor, Tensor]:
+    return ops.attn_fwd(query, key, value, softmax_scale=softmax_scale, q_descale=q_descale,
+                        k_descale=k_descale, v_descale=v_descale,
+                        out_dtype=torch.float16 if out_fp16 else torch.bfloat16)
+
+
+@register_fake("xdit_amd::attn_fwd_fp8")
+def _attn_fwd_fp8_fake(query, key, value, q_descale, k_descale, v_descale, softmax_scale, out_fp16):
+    return _fake_out_lse(query, torch.float16 if out_fp16 else torch.bfloat16)
+
+
+@custom_op("xdit_amd::lse_merge", mutates_args=("acc_out", "acc_lse"), device_types="cuda")
+def lse_merge(acc_out: Tensor, acc_lse: Tensor, block_out: Tensor, block_lse: Tensor, first: bool) -> None:
+    ops.lse_merge(acc_out, acc_lse, block_out, block_lse, first=first)
+
+
+@register_fake("xdit_amd::lse_merge")
+def _lse_merge_fake(acc_out, acc_lse, block_out, block_lse, first):
+    return None
+
+
+@custom_op("xdit_amd::lse_merge_final", mutates_args=("acc_out", "acc_lse", "final_out"), device_types="cuda")
+def lse_merge_final(acc_out: Tensor, acc_lse: Tensor, block_out: Tensor, block_lse: Tensor, final_out: Tensor) -> None:
+    ops.lse_merge(acc_out, acc_lse, block_out, block_lse, first=False, final_out=final_out)
+
+
+@register_fake("xdit_amd::lse_merge_final")
+def _lse_merge_final_fake(acc_out, acc_lse, block_out, block_lse, final_out):
+    return None
+
+
+@custom_op("xdit_amd::fp8_quant", mutates_args=(), device_types="cuda")
+def fp8_quant(x: Tensor, per_tensor: bool) -> Tuple[Tensor, Tensor]:
+    return ops.fp8_quant(x, per_tensor=per_tensor)
+
+
+@register_fake("xdit_amd::fp8_quant")
+def _fp8_quant_fake(x, per_tensor):
+    B, H, S, D = x.shape
+    return (x.new_empty((B, H, S, D), dtype=torch.float8_e4m3fn),
+            x.new_empty((B, H), dtype=torch.float32))

@@ -20,6 +20,11 @@ _DEFAULT_BACKEND = AttentionBackendType.MI355
 def set_default_backend(backend):
     """Counterpart of RuntimeState.set_attention_backend (runtime_state.py:113-131)."""
     global _DEFAULT_BACKEND
+    if isinstance(backend, str):
+        try:
+            backend = AttentionBackendType[backend.upper()]
+        except KeyError:
+            raise ValueError(f"Value '{backend}' is not a valid attention backend.") from None
     if backend not in ATTENTION_FUNCTION_REGISTRY:
         raise NotImplementedError(f"Attention backend {backend} not registered.")
     _DEFAULT_BACKEND = backend
