@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define XDIT_ATTN_ABI_VERSION 2
+#define XDIT_ATTN_ABI_VERSION 3
 
 typedef enum {
   XDIT_OK = 0,
@@ -149,6 +149,12 @@ int xdit_lse_merge(const xdit_merge_args* args);
  * `scale_in != NULL` (device pointer to one float) supplies a static scale instead of the abs-max
  * (the `scale=` argument of per_tensor_quant).  Values whose quotient exceeds 448 saturate.
  * `descale` (B*H contiguous fp32) doubles as the reduction buffer; no other memory is used.
+ * `hadamard_block` (0 or 1 = off; else a power of two <= 128 that divides D) first rotates every
+ * row along head_dim, block by block, by the orthonormal Sylvester-Hadamard matrix R of that size
+ * with entries +-r, r = 1/sqrt(block) rounded to in_dtype, and rounds the result to in_dtype:
+ * `torch.matmul(x.unflatten(-1, (D/block, block)), R).flatten(-2)` of the reference's
+ * _fp8_hadamard_rotate (attention_backend.py:703-714; matrix :71-94).  Applied to both q and k
+ * it leaves q.k unchanged and spreads outliers before the fp8 cast (:725-728).
  */
 typedef struct {
   uint32_t struct_size;        /* = sizeof(xdit_quant_args) */
@@ -162,6 +168,8 @@ typedef struct {
   const float* scale_in;       /* optional static scale, may be NULL */
   xdit_strides x_stride, y_stride;
   void* stream;
+  int32_t hadamard_block;
+  int32_t reserved0;
 } xdit_quant_args;
 
 int xdit_fp8_quant(const xdit_quant_args* args);

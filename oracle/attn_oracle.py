@@ -19,13 +19,17 @@ which is the PyTorch wheel the reference depends on):
                          in the order a rank would receive them), joint K/V on the first ("front")
                          or last ("rear") step, :89-100.
 * `per_tensor_quant_ref` attention_backend.py:606-615.
+* `hadamard_matrix`, `hadamard_rotate_ref`  attention_backend.py:71-94 (Sylvester construction,
+                         1/sqrt(n) normalisation) and :703-714 (block-wise rotation of head_dim).
 * `sdpa_cpu`             the body of `_sdpa_attn_call`, attention_backend.py:499-501 (used as the
                          timed CPU baseline).
 
 Pinning (tests/test_oracle.py): brute force with math.fsum on tiny inputs; torch's own CPU
 ops `aten._scaled_dot_product_attention_math` and `aten._scaled_dot_product_flash_attention_for_cpu`;
 closed forms and invariants of the merge (log-add-exp identity, fold of any KV partition equals the
-single pass, -inf block is the identity, equal lse gives the mean); the C twin in attn_ref.c.
+single pass, -inf block is the identity, equal lse gives the mean); the C twin in attn_ref.c;
+for the Hadamard rotation the sign rule (-1)^popcount(i&j), orthonormality, an independent fast
+Walsh-Hadamard transform, and invariance of q.k under a common rotation.
 The reference holds no golden vectors for this path, so values are pinned by those checks, and
 the tolerances (not values) come from the reference's tests.
 """
@@ -182,6 +186,27 @@ def per_head_quant_ref(x):
     scale = torch.where(amax > 0, amax / FP8_MAX, torch.ones_like(amax))
     y = (x / scale[:, :, None, None]).to(torch.float8_e4m3fn)
     return y, scale
+
+
+def hadamard_matrix(block_r, dtype=torch.float64):
+    """Orthonormal Sylvester-Hadamard matrix: H1=[[1]], H2n=[[Hn,Hn],[Hn,-Hn]], divided by
+    sqrt(block_r) in float32 and then cast to `dtype` (attention_backend.py:86-94, the construction
+    the reference falls back to and the normalisation it applies at :85)."""
+    assert block_r > 0 and (block_r & (block_r - 1)) == 0
+    H = torch.ones((1, 1), dtype=torch.float32)
+    while H.shape[0] < block_r:
+        H = torch.cat([torch.cat([H, H], dim=1), torch.cat([H, -H], dim=1)], dim=0)
+    return (H / (block_r ** 0.5)).to(dtype)
+
+
+def hadamard_rotate_ref(x, block_r):
+    """_fp8_hadamard_rotate (attention_backend.py:703-714): x @ R along head_dim in blocks of
+    block_r, R held in x's dtype, result in x's dtype.  The products are summed in float64 here
+    (a matmul sums them in fp32 in an unspecified order), then rounded once to x's dtype."""
+    d = x.shape[-1]
+    R = hadamard_matrix(block_r, x.dtype).to(torch.float64)
+    xb = x.to(torch.float64).unflatten(-1, (d // block_r, block_r))
+    return torch.matmul(xb, R).flatten(-2).to(x.dtype)
 
 
 def dequant(y, scale):

@@ -376,6 +376,58 @@ def test_fp8_quant_bit_exact(gpu, dtype):
     assert d0.item() == 1.0 and torch.all(y0.float() == 0)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("block,D", [(128, 128), (32, 128), (8, 64), (2, 128), (64, 64), (16, 96)])
+def test_fp8_quant_with_hadamard_rotation(gpu, dtype, block, D):
+    """Rotation fused into the quantiser against rotate-then-quantise on the oracle.  The kernel
+    sums the +-x terms in fp32 in butterfly order, the oracle in float64, so a value that lands
+    within fp32 rounding of a rounding boundary of `dtype` (and then of fp8) may differ by one
+    step: at most 1 % of the bytes may differ and then only by one fp8 step; scales may differ by
+    one step of `dtype`."""
+    g = torch.Generator().manual_seed(block + D)
+    x = torch.randn(2, 3, 77, D, generator=g)
+    x[0, 1, 5, 3] = 40.0  # an outlier
+    x = x.to(dtype)
+    y, d = ops.fp8_quant(_layout(x, "bshd", gpu), hadamard_block=block)
+    rot = O.hadamard_rotate_ref(x, block)
+    ry, rd = O.per_head_quant_ref(rot)
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -22}[dtype]
+    assert torch.allclose(d.cpu(), rd, rtol=2 * eps, atol=0)
+    a, b = y.cpu().view(torch.uint8).int(), ry.view(torch.uint8).int()
+    assert (a != b).float().mean().item() <= 0.01
+    assert ((a - b).abs() <= 1).all()
+    # rotating back (R is symmetric and orthonormal) recovers x to fp8 accuracy
+    back = O.hadamard_rotate_ref(O.dequant(y.cpu(), d.cpu()).double(), block)
+    assert (back - x.double()).abs().max().item() <= 2.0 ** -4 * x.double().abs().max().item()
+    with pytest.raises(ValueError):
+        ops.fp8_quant(x.to(gpu), hadamard_block=48)
+    with pytest.raises(ValueError):
+        ops.fp8_quant(x.to(gpu), hadamard_block=256)
+
+
+@pytest.mark.parametrize("outlier", [1.0, 12.0])
+def test_fp8_adapter_rotation(gpu, outlier):
+    """The fp8 adapter with q and k rotated inside the quantiser (q.k is invariant under a common
+    rotation) against the attention of the UNQUANTISED inputs.  Without outliers both forms stay
+    within the fp8 tolerance; with one channel of q and k 12x larger (which per-tensor fp8
+    quantisation resolves badly) the rotation must cut the error by more than half."""
+    q, k, v = O.make_qkv(1, 4, 640, 128, seed=71, dtype=torch.float32)
+    q[..., 7] *= outlier
+    k[..., 7] *= outlier
+    s = 1.0 if outlier == 1.0 else 0.3
+    q, k, v = (t.to(torch.bfloat16) for t in (q * s, k * s, v))
+    ro, rl = O.attn_fwd_ref(q, k, v)
+    fn = AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355_FP8]
+    o_rot, l_rot = fn(q.to(gpu), k.to(gpu), v.to(gpu), 0.0, False)
+    o_off, l_off = fn(q.to(gpu), k.to(gpu), v.to(gpu), 0.0, False, attention_kwargs={"hadamard_block": 0})
+    assert AB.FP8_HADAMARD_BLOCK == 128 and not torch.equal(o_rot, o_off)
+    if outlier == 1.0:
+        assert _err(o_rot, ro) <= 6e-2 and _err(o_off, ro) <= 6e-2
+        assert _err(l_rot, rl) <= 5e-2 and _err(l_off, rl) <= 5e-2
+    else:
+        assert _err(o_rot, ro) <= 0.5 * _err(o_off, ro) and _err(l_rot, rl) <= 0.5 * _err(l_off, rl)
+
+
 # ---------------------------------------------------------------------------- call surfaces
 @pytest.mark.parametrize("strategy", ["front", "rear"])
 @pytest.mark.parametrize("chunks", [1, 2])
@@ -407,7 +459,7 @@ def test_fp8_backend_adapter(gpu):
     q, k, v = O.make_qkv(1, 4, 512, 128, seed=51, dtype=torch.bfloat16)
     ro, rl = O.attn_fwd_ref(q, k, v)
     o, l = AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355_FP8](q.to(gpu), k.to(gpu), v.to(gpu), 0.0, False)
-    assert o.dtype == torch.bfloat16 and _err(o, ro) <= 6e-2 and _err(l, rl) <= 2e-2
+    assert o.dtype == torch.bfloat16 and _err(o, ro) <= 6e-2 and _err(l, rl) <= 5e-2  # vs the UNQUANTISED inputs
     assert torch.equal(o, usp.attention(q.to(gpu), k.to(gpu), v.to(gpu), backend=AB.AttentionBackendType.MI355_FP8))
 
 
@@ -436,7 +488,7 @@ def test_custom_ops_opcheck_and_compile(gpu):
     tests = ("test_schema", "test_faketensor", "test_autograd_registration")
     torch.library.opcheck(torch.ops.xdit_amd.attn_fwd.default, (q, k, v, 128 ** -0.5), test_utils=tests)
     torch.library.opcheck(torch.ops.xdit_amd.attn_fwd_joint.default, (q, k, v, jk, jv, 128 ** -0.5), test_utils=tests)
-    torch.library.opcheck(torch.ops.xdit_amd.fp8_quant.default, (q, True), test_utils=tests)
+    torch.library.opcheck(torch.ops.xdit_amd.fp8_quant.default, (q, True, 128), test_utils=tests)
     o, l = ops.attn_fwd(q, k, v)
     acc_o, acc_l = o.float(), l.clone()
     torch.library.opcheck(torch.ops.xdit_amd.lse_merge.default, (acc_o, acc_l, o, l, False), test_utils=tests)

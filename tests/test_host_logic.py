@@ -140,7 +140,7 @@ def test_custom_ops_fake_implementations_describe_the_outputs():
     assert out.dtype == torch.float16 and out.shape == (B, H, Sq, D) and lse.dtype == torch.float32
     out, _ = torch.ops.xdit_amd.attn_fwd_fp8(q8, k8, k8, d, d, d, 0.1, False)
     assert out.dtype == torch.bfloat16
-    y, ds = torch.ops.xdit_amd.fp8_quant(q, False)
+    y, ds = torch.ops.xdit_amd.fp8_quant(q, False, 128)
     assert y.dtype == torch.float8_e4m3fn and y.shape == q.shape and y.is_contiguous() and ds.shape == (B, H)
     # there is no CPU implementation behind the ops either
     with pytest.raises((NotImplementedError, RuntimeError)):

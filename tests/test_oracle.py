@@ -224,3 +224,59 @@ def test_c1_golden_fixture_against_oracle_and_torch():
     assert np.allclose(l.numpy(), z["lse"], atol=1e-6)
     mo, _ = torch.ops.aten._scaled_dot_product_attention_math(c1["q"], c1["k"], c1["v"])
     assert np.allclose(mo[:, :, ::37].numpy(), z["out_rows"], atol=5e-6)
+
+
+# ---------------------------------------------------------------------------- Hadamard rotation
+@pytest.mark.parametrize("n", [1, 2, 8, 32, 128])
+def test_hadamard_matrix_sign_rule_and_orthonormality(n):
+    """Sylvester's matrix has entries (-1)^popcount(i & j); scaled by 1/sqrt(n) it is symmetric
+    and orthonormal.  A transposed block or a wrong sign in the recursion fails the sign rule."""
+    R = O.hadamard_matrix(n)
+    i = torch.arange(n)
+    pop = torch.tensor([[bin(int(a) & int(b)).count("1") for b in i] for a in i])
+    expect = torch.where(pop % 2 == 0, 1.0, -1.0).double() * float(torch.tensor(1.0) / torch.tensor(n ** 0.5))
+    assert torch.allclose(R, expect, atol=1e-7)
+    assert torch.allclose(R @ R.T, torch.eye(n, dtype=torch.float64), atol=1e-6)
+    assert torch.equal(R, R.T)
+
+
+def _fwht(x):
+    """Textbook in-place fast Walsh-Hadamard transform (natural order), pure Python."""
+    x = list(x)
+    h = 1
+    while h < len(x):
+        for i in range(0, len(x), 2 * h):
+            for j in range(i, i + h):
+                x[j], x[j + h] = x[j] + x[j + h], x[j] - x[j + h]
+        h *= 2
+    return x
+
+
+@pytest.mark.parametrize("block", [8, 32, 128])
+def test_hadamard_rotate_ref_against_fwht_and_invariance(block):
+    g = torch.Generator().manual_seed(block)
+    x = torch.randn(1, 2, 5, 128, generator=g, dtype=torch.float64)
+    y = O.hadamard_rotate_ref(x, block)
+    r = float(torch.tensor(1.0) / torch.tensor(block ** 0.5))  # the fp32 normalisation the reference applies
+    for row in (0, 3):
+        for b0 in range(0, 128, block):
+            ref = [v * r for v in _fwht(x[0, 1, row, b0:b0 + block].tolist())]
+            assert torch.allclose(y[0, 1, row, b0:b0 + block], torch.tensor(ref, dtype=torch.float64), atol=1e-12)
+    # rotating q and k alike leaves the logits unchanged (up to the fp32 rounding of 1/sqrt(n))
+    k = torch.randn(1, 2, 7, 128, generator=g, dtype=torch.float64)
+    s0 = x @ k.transpose(-1, -2)
+    s1 = y @ O.hadamard_rotate_ref(k, block).transpose(-1, -2)
+    assert torch.allclose(s0, s1, rtol=1e-6, atol=1e-6)
+    # bf16: result is the correctly rounded product with the matrix held in bf16
+    xb = x.to(torch.bfloat16)
+    yb = O.hadamard_rotate_ref(xb, block)
+    assert yb.dtype == torch.bfloat16
+    Rb = O.hadamard_matrix(block, torch.bfloat16).double()
+    blk = xb.double()[..., :block] @ Rb
+    assert torch.equal(yb[..., :block], blk.to(torch.bfloat16))
+    # an outlier is spread evenly over its block
+    e = torch.zeros(1, 1, 1, 128, dtype=torch.float64)
+    e[..., 5] = 64.0
+    ye = O.hadamard_rotate_ref(e, block)
+    assert torch.allclose(ye[..., :block].abs(), torch.full((block,), 64.0 * r, dtype=torch.float64))
+    assert (ye[..., block:] == 0).all() or block == 128

@@ -9,7 +9,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libxdit_amd_attn.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 XDIT_OK = 0
 XDIT_ERR_INVALID_ARG = -1
@@ -105,6 +105,8 @@ class QuantArgs(ctypes.Structure):
         ("x_stride", Strides),
         ("y_stride", Strides),
         ("stream", ctypes.c_void_p),
+        ("hadamard_block", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
     ]
 
 

@@ -84,22 +84,33 @@ def get_dtype_max(dtype):
         return torch.iinfo(dtype).max
 
 
-def per_tensor_quant(x, scale=None, scale_dtype=torch.float32, quant_dtype=torch.float8_e4m3fn, dtypeMax=None):
+# Block size of the Hadamard rotation the fp8 adapter applies to q and k before quantising, as the
+# reference's AITER fp8 adapter does with a 128x128 matrix (attention_backend.py:374, :725-728).
+# 0 switches it off (the reference's FLASH_3_FP8 adapter, :617-642, does not rotate).
+FP8_HADAMARD_BLOCK = 128
+
+
+def per_tensor_quant(x, scale=None, scale_dtype=torch.float32, quant_dtype=torch.float8_e4m3fn, dtypeMax=None,
+                     hadamard_block=0):
     """Same contract as the reference's per_tensor_quant (attention_backend.py:606-615):
     one abs-max scale over the whole tensor, y = fp8(x / scale), descale expanded to x.shape[:2].
-    With `scale=None` the abs-max reduction and the cast run in the HIP quantiser."""
+    With `scale=None` the abs-max reduction and the cast run in the HIP quantiser.
+    `hadamard_block` fuses _fp8_hadamard_rotate (:703-714) in front: x is rotated along head_dim
+    in blocks of that size before the abs-max and the cast."""
     if quant_dtype != torch.float8_e4m3fn:
         raise NotImplementedError("only float8_e4m3fn (the fp8 format of gfx950) is supported")
     if scale is None and dtypeMax in (None, get_dtype_max(quant_dtype)):
         if torch.compiler.is_compiling():
-            y, descale = torch.ops.xdit_amd.fp8_quant(x, True)
+            y, descale = torch.ops.xdit_amd.fp8_quant(x, True, hadamard_block)
         else:
-            y, descale = ops.fp8_quant(x, per_tensor=True)
+            y, descale = ops.fp8_quant(x, per_tensor=True, hadamard_block=hadamard_block)
         return y, descale.to(scale_dtype)
     if scale is None:
+        if hadamard_block > 1:
+            raise NotImplementedError("a non-default dtypeMax together with the fused rotation is not implemented")
         scale = torch.abs(x.to(torch.float32)).max() / dtypeMax
     scale = torch.as_tensor(scale, dtype=torch.float32, device=x.device)
-    y, descale = ops.fp8_quant(x, per_tensor=True, scale=scale)
+    y, descale = ops.fp8_quant(x, per_tensor=True, scale=scale, hadamard_block=hadamard_block)
     return y, descale.to(scale_dtype)
 
 
@@ -108,6 +119,8 @@ def _mi355_fp8_attn_call(query, key, value, dropout_p, is_causal, attention_kwar
     """fp8 attention: quantise q, k, v per tensor (as _flash_attn_3_fp8_call :617-642 and
     _aiter_fp8_attn_call :717-772 do), run the fp8 kernel with (B,H) descales, return a bf16/fp16
     output in the query's dtype AND the lse (the reference's AITER fp8 path returns no lse, :732).
+    q and k are Hadamard-rotated along head_dim inside the quantiser (block FP8_HADAMARD_BLOCK, or
+    attention_kwargs["hadamard_block"]; 0 = off), as the AITER fp8 adapter does (:725-728).
     Inputs that are already float8_e4m3fn take their descales from attention_kwargs
     ("q_descale", "k_descale", "v_descale")."""
     _check_call(dropout_p, is_causal, attention_kwargs)
@@ -121,8 +134,12 @@ def _mi355_fp8_attn_call(query, key, value, dropout_p, is_causal, attention_kwar
                             k_descale=kw.get("k_descale"), v_descale=kw.get("v_descale"),
                             out_dtype=kw.get("out_dtype", torch.bfloat16))
     out_dtype = query.dtype if query.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
-    q8, qd = per_tensor_quant(query)
-    k8, kd = per_tensor_quant(key)
+    had = (attention_kwargs or {}).get("hadamard_block", FP8_HADAMARD_BLOCK)
+    if had > 1 and query.shape[-1] % had != 0:
+        had = 0
+    # rotating q and k alike leaves q.k unchanged and spreads outliers before the fp8 cast
+    q8, qd = per_tensor_quant(query, hadamard_block=had)
+    k8, kd = per_tensor_quant(key, hadamard_block=had)
     v8, vd = per_tensor_quant(value)
     if torch.compiler.is_compiling():
         return torch.ops.xdit_amd.attn_fwd_fp8(q8, k8, v8, qd, kd, vd, scale, out_dtype == torch.float16)

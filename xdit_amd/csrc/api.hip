@@ -221,8 +221,13 @@ int xdit_fp8_quant(const xdit_quant_args* a) {
   if ((reinterpret_cast<uintptr_t>(a->y) & 7u) || a->y_stride.b % 8 || a->y_stride.h % 8 || a->y_stride.s % 8)
     return fail(XDIT_ERR_INVALID_ARG, "y must be 8-byte aligned with strides that are multiples of 8");
   if (a->y_stride.s < a->D) return fail(XDIT_ERR_INVALID_ARG, "y: S stride smaller than head_dim");
+  const int hb = a->hadamard_block;
+  if (hb < 0 || hb > 128 || (hb & (hb - 1)) != 0 || (hb > 1 && a->D % hb != 0))
+    return fail(XDIT_ERR_INVALID_ARG, "hadamard_block %d must be 0 or a power of two <= 128 that divides head_dim %d", hb, a->D);
   xdit::QuantParams p;
   std::memset(&p, 0, sizeof(p));
+  p.had_block = hb > 1 ? hb : 0;
+  p.had_scale = hb > 1 ? 1.0f / std::sqrt((float)hb) : 1.0f;
   p.x = a->x; p.y = a->y; p.amax = a->descale; p.descale = a->descale; p.scale_in = a->scale_in;
   p.xs_b = a->x_stride.b; p.xs_h = a->x_stride.h; p.xs_s = a->x_stride.s;
   p.ys_b = a->y_stride.b; p.ys_h = a->y_stride.h; p.ys_s = a->y_stride.s;

@@ -7,7 +7,8 @@
 // in a HIP graph), (2) abs-max reduction with one atomic max per workgroup, (3) scale and cast,
 // (4) turn the abs-max buffer into the descale values.  Both tensor passes are HBM-bound and read
 // 16 bytes per lane; the division is a true fp32 division so results match the reference's
-// `x / scale` bit for bit.
+// `x / scale` bit for bit.  Optionally both passes first rotate each row along head_dim by a
+// block Hadamard matrix (_fp8_hadamard_rotate, attention_backend.py:703-714), in registers.
 #include "common.h"
 #include "launchers.h"
 
@@ -31,6 +32,42 @@ template <> __device__ __forceinline__ void load8<_Float16>(const _Float16* p, f
   for (int i = 0; i < 8; i++) x[i] = (float)v[i];
 }
 
+// Rotates the rows by the Sylvester-Hadamard matrix of size `block` along head_dim, in place in
+// the 8-element chunks the threads hold: the three butterfly levels inside a chunk in
+// registers, the levels across chunks by exchanging with the lane that holds chunk c ^ m of the
+// same row (the chunks of a block sit in consecutive, block-aligned lanes of one wavefront).
+// Entries are +-r with r = `scale` rounded to T and the result is rounded to T, like the output
+// of a matmul with the matrix held in T.  `c` is the chunk's index within its row.
+template <typename T>
+__device__ __forceinline__ void hadamard_rows(float (&v)[8], int block, float scale, int c) {
+  if (block >= 2) {
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) { const float a = v[j], b = v[j + 1]; v[j] = a + b; v[j + 1] = a - b; }
+  }
+  if (block >= 4) {
+#pragma unroll
+    for (int j = 0; j < 8; j += 4) {
+#pragma unroll
+      for (int i = 0; i < 2; i++) { const float a = v[j + i], b = v[j + i + 2]; v[j + i] = a + b; v[j + i + 2] = a - b; }
+    }
+  }
+  if (block >= 8) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) { const float a = v[i], b = v[i + 4]; v[i] = a + b; v[i + 4] = a - b; }
+  }
+  for (int m = 1; m * 8 < block; m <<= 1) {
+    const bool upper = (c & m) != 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float o = __shfl_xor(v[j], m);
+      v[j] = upper ? o - v[j] : v[j] + o;
+    }
+  }
+  const float r = (float)(T)scale;
+#pragma unroll
+  for (int j = 0; j < 8; j++) v[j] = (float)(T)(v[j] * r);
+}
+
 __global__ void fill_zero_kernel(float* p, int n) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0.f;
@@ -50,6 +87,7 @@ __global__ __launch_bounds__(256) void absmax_kernel(const QuantParams p) {
     const int c = (int)(i - s * cpr);
     float v[8];
     load8<T>(x + s * p.xs_s + c * 8, v);
+    if (p.had_block > 1) hadamard_rows<T>(v, p.had_block, p.had_scale, c);
 #pragma unroll
     for (int j = 0; j < 8; j++) m = fmaxf(m, fabsf(v[j]));  // fmaxf drops NaN operands
   }
@@ -85,6 +123,7 @@ __global__ __launch_bounds__(256) void cast_kernel(const QuantParams p) {
     const int c = (int)(i - s * cpr);
     float v[8];
     load8<T>(x + s * p.xs_s + c * 8, v);
+    if (p.had_block > 1) hadamard_rows<T>(v, p.had_block, p.had_scale, c);
 #pragma unroll
     for (int j = 0; j < 8; j++) v[j] = v[j] / scale;
     int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);

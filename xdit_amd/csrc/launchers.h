@@ -36,6 +36,8 @@ struct QuantParams {
   int64_t ys_b, ys_h, ys_s;
   int B, H, S, D;
   int per_tensor;
+  int had_block;    // Hadamard rotation block along head_dim (<= 1: none)
+  float had_scale;  // 1/sqrt(had_block) in fp32; the kernel rounds it to the input dtype
 };
 
 // dtype codes below are the C ABI's xdit_dtype values: 0 bf16, 1 fp16, 2 fp32, 3 fp8 e4m3fn.

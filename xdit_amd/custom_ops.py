@@ -11,7 +11,7 @@ The reference wraps a vendor kernel the same way (xfuser/core/distributed/attent
                                softmax_scale, out_fp16)                     -> (out, lse)
     xdit_amd::lse_merge       (acc_out, acc_lse, block_out, block_lse, first)   in place
     xdit_amd::lse_merge_final (acc_out, acc_lse, block_out, block_lse, final_out)  in place
-    xdit_amd::fp8_quant       (x, per_tensor)                               -> (y, descale)
+    xdit_amd::fp8_quant       (x, per_tensor, hadamard_block)               -> (y, descale)
 
 All tensors are logical BHSD (any B/H/S strides); outputs are BHSD-contiguous, lse is (B,H,Sq)
 fp32.  The ops are registered for GPU tensors only: there is no CPU implementation.
@@ -87,12 +87,12 @@ def _lse_merge_final_fake(acc_out, acc_lse, block_out, block_lse, final_out):
 
 
 @custom_op("xdit_amd::fp8_quant", mutates_args=(), device_types="cuda")
-def fp8_quant(x: Tensor, per_tensor: bool) -> Tuple[Tensor, Tensor]:
-    return ops.fp8_quant(x, per_tensor=per_tensor)
+def fp8_quant(x: Tensor, per_tensor: bool, hadamard_block: int) -> Tuple[Tensor, Tensor]:
+    return ops.fp8_quant(x, per_tensor=per_tensor, hadamard_block=hadamard_block)
 
 
 @register_fake("xdit_amd::fp8_quant")
-def _fp8_quant_fake(x, per_tensor):
+def _fp8_quant_fake(x, per_tensor, hadamard_block):
     B, H, S, D = x.shape
     return (x.new_empty((B, H, S, D), dtype=torch.float8_e4m3fn),
             x.new_empty((B, H), dtype=torch.float32))

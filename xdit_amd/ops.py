@@ -175,10 +175,11 @@ def lse_merge(acc_out, acc_lse, block_out, block_lse, first=False, final_out=Non
     return acc_out, acc_lse
 
 
-def fp8_quant(x, per_tensor=False, scale=None):
+def fp8_quant(x, per_tensor=False, scale=None, hadamard_block=0):
     """Abs-max fp8 quantiser on a logical BHSD tensor -> (y float8_e4m3fn BHSD-contiguous,
     descale (B,H) fp32).  `per_tensor` takes one abs-max over the whole tensor (the reference's
-    per_tensor_quant); `scale` (a one-element fp32 tensor) is a static scale."""
+    per_tensor_quant); `scale` (a one-element fp32 tensor) is a static scale; `hadamard_block`
+    (a power of two dividing head_dim) rotates the rows by a block Hadamard matrix first."""
     device = x.device
     _check4("x", x, device)
     B, H, S, D = x.shape
@@ -188,6 +189,7 @@ def fp8_quant(x, per_tensor=False, scale=None):
     a.struct_size = ctypes.sizeof(_lib.QuantArgs)
     a.in_dtype = _code(x.dtype)
     a.per_tensor = 1 if per_tensor else 0
+    a.hadamard_block = int(hadamard_block)
     a.B, a.H, a.D, a.S = B, H, D, S
     a.x, a.y, a.descale = x.data_ptr(), y.data_ptr(), descale.data_ptr()
     if scale is not None:
