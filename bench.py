@@ -13,7 +13,8 @@ q/k per-head RMSNorm'd), inputs resident in HBM.  Prints ONE JSON line:
                xfuser/core/distributed/attention_backend.py:499-501) on a bounded sample of the
                same workload, timed on this host's cores
   also         the other named shapes: HunyuanVideo-720p head shard (bf16), Wan2.1 720p head
-               shard (fp8), the 4-chunk ring with its fp32 merges, the merge kernel's GB/s
+               shard (fp8), the 4-chunk ring with its fp32 merges, the merge kernel's GB/s, the
+               fp8 quantiser and the fused norm + rotary prologue (GB/s against the HBM peak)
 Everything runs on one GPU; --gpus above 1 is refused (this build has no multi-GPU path).
 """
 import argparse
@@ -207,6 +208,20 @@ def main():
         _, ms = time_calls(lambda: ops.fp8_quant(qw), 10, 2)
         also["fp8_quant_wan_shard"] = {"us": round(ms * 1e3, 1), "gbs": round(qw.numel() * 5.0 / ms / 1e6, 1)}
         del qw, kw, vw, q8, k8, v8
+        # pre-attention prologue (per-head RMSNorm + rotary embedding + BSHD -> BHSD), bf16:
+        # bytes per call = 4*N*D (read + write) + 8*S*D (cos and sin rows, read once)
+        from xdit_amd import prologue
+        for name, (Bp, Sp, Hp) in (("prologue_flux_q", (1, 4608, 24)), ("prologue_hunyuan_q", (1, 119056, 24))):
+            xp = torch.randn(Bp, Sp, Hp, D, device=dev).bfloat16()
+            wp = torch.ones(D, device=dev).bfloat16()
+            ang = torch.rand(Sp, D, device=dev)
+            cs, sn = ang.cos(), ang.sin()
+            yp = torch.empty(Bp, Hp, Sp, D, device=dev, dtype=torch.bfloat16)
+            _, ms = time_calls(lambda: prologue.norm_rope(xp, weight=wp, freqs_cis=(cs, sn), sequence_dim=1, out=yp), 20, 3)
+            pbytes = 4.0 * xp.numel() + 8.0 * Sp * D
+            also[name] = {"us": round(ms * 1e3, 2), "gbs": round(pbytes / ms / 1e6, 1),
+                          "frac_hbm_peak": round(pbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": pbytes}
+            del xp, yp, ang, cs, sn
         result["also"] = also
 
     if args.copy_calibration:

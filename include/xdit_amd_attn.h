@@ -174,6 +174,53 @@ typedef struct {
 
 int xdit_fp8_quant(const xdit_quant_args* args);
 
+/*
+ * Pre-attention prologue of an xDiT attention processor, fused into one pass over Q (or K):
+ *     y = rotary(norm(x)), written through its own strides (e.g. BSHD in, BHSD-contiguous out)
+ * replacing `attn.norm_q(query)`, `apply_rotary_emb(query, image_rotary_emb)` and the later
+ * `.transpose(1, 2)` + contiguous copy (transformer_flux.py:116-147,
+ * transformer_hunyuan_video.py:48-83, transformer_wan.py:99-122 under
+ * xfuser/model_executor/models/transformers/).  With norm and rotation off it is a strided
+ * re-layout (what V needs).  x and y are logical (B,H,S,D) with element strides.
+ *   norm   XDIT_NORM_NONE; XDIT_NORM_HEAD: RMSNorm over head_dim of every (b,h,s) row, `weight`
+ *          has D entries; XDIT_NORM_TOKEN: over all H*D elements of a token, `weight` has H*D
+ *          entries indexed h*D+d (Wan's norm over the un-split projection).  Statistics in fp32:
+ *          x * rsqrt(mean(x^2) + eps), rounded to dtype, times weight (same dtype; NULL = no
+ *          gain), rounded again: the roundings of diffusers' RMSNorm with a 16-bit gain.
+ *   rope   XDIT_ROPE_NONE; XDIT_ROPE_INTERLEAVED: pairs (2i, 2i+1),
+ *          out[j] = x[j] cos[j] + rot[j] sin[j] with rot = (-x[2i+1], x[2i]) (diffusers
+ *          apply_rotary_emb, use_real_unbind_dim=-1); XDIT_ROPE_SPLIT_HALF: pairs (j, j + D/2)
+ *          (use_real_unbind_dim=-2); XDIT_ROPE_WAN: out[2i] = x[2i] cos[2i] - x[2i+1] sin[2i+1],
+ *          out[2i+1] = x[2i] sin[2i+1] + x[2i+1] cos[2i] (transformer_wan.py:108-120).
+ *          cos / sin are fp32, `rope_stride` elements from row to row, D values per row, shared
+ *          by batch and heads.  Only sequence rows [rope_row0, rope_row0 + rope_rows) are
+ *          rotated, with table row s - rope_row0 (HunyuanVideo rotates the video tokens and not
+ *          the text tokens behind them); products in fp32, result rounded to dtype.
+ */
+enum xdit_norm_mode { XDIT_NORM_NONE = 0, XDIT_NORM_HEAD = 1, XDIT_NORM_TOKEN = 2 };
+enum xdit_rope_mode { XDIT_ROPE_NONE = 0, XDIT_ROPE_INTERLEAVED = 1, XDIT_ROPE_SPLIT_HALF = 2, XDIT_ROPE_WAN = 3 };
+
+typedef struct {
+  uint32_t struct_size;        /* = sizeof(xdit_prologue_args) */
+  int32_t dtype;               /* bf16, fp16 or fp32: x, y and weight */
+  int32_t norm;                /* xdit_norm_mode */
+  int32_t rope;                /* xdit_rope_mode */
+  int32_t B, H, D;
+  float eps;
+  int64_t S;
+  const void* x;
+  void* y;
+  const void* weight;          /* may be NULL */
+  const float* cos;            /* NULL when rope == XDIT_ROPE_NONE */
+  const float* sin;
+  int64_t rope_stride;
+  int64_t rope_row0, rope_rows;
+  xdit_strides x_stride, y_stride;
+  void* stream;
+} xdit_prologue_args;
+
+int xdit_qk_prologue(const xdit_prologue_args* args);
+
 /* Message of the last error on the calling thread ("" if none). Never NULL. */
 const char* xdit_attn_last_error(void);
 

@@ -21,6 +21,10 @@ which is the PyTorch wheel the reference depends on):
 * `per_tensor_quant_ref` attention_backend.py:606-615.
 * `hadamard_matrix`, `hadamard_rotate_ref`  attention_backend.py:71-94 (Sylvester construction,
                          1/sqrt(n) normalisation) and :703-714 (block-wise rotation of head_dim).
+* `rms_norm_ref`, `apply_rotary_emb_ref`, `apply_rotary_emb_wan_ref`  the steps of the attention
+                         processors in front of the attention call: transformer_flux.py:116-147,
+                         transformer_hunyuan_video.py:48-83, transformer_wan.py:99-122.  The first two
+                         restate diffusers (>=0.33.0, absent here) from its published source.
 * `sdpa_cpu`             the body of `_sdpa_attn_call`, attention_backend.py:499-501 (used as the
                          timed CPU baseline).
 
@@ -29,7 +33,10 @@ ops `aten._scaled_dot_product_attention_math` and `aten._scaled_dot_product_flas
 closed forms and invariants of the merge (log-add-exp identity, fold of any KV partition equals the
 single pass, -inf block is the identity, equal lse gives the mean); the C twin in attn_ref.c;
 for the Hadamard rotation the sign rule (-1)^popcount(i&j), orthonormality, an independent fast
-Walsh-Hadamard transform, and invariance of q.k under a common rotation.
+Walsh-Hadamard transform, and invariance of q.k under a common rotation; for the prologue
+torch's own `F.rms_norm` in float64, complex multiplication as the independent form of the
+rotation, pair-norm preservation, identity at angle 0, and agreement of the three rotation
+conventions on tables where they must agree.
 The reference holds no golden vectors for this path, so values are pinned by those checks, and
 the tolerances (not values) come from the reference's tests.
 """
@@ -212,6 +219,85 @@ def hadamard_rotate_ref(x, block_r):
 def dequant(y, scale):
     """fp8 bytes + (B,H) scales -> float32 BHSD."""
     return y.to(torch.float32) * scale[:, :, None, None].to(torch.float32)
+
+
+# ----------------------------------------------------------------------------------------------
+# pre-attention prologue (RMSNorm of Q/K, rotary embedding)
+# ----------------------------------------------------------------------------------------------
+def rms_norm_ref(x, weight=None, eps=1e-6):
+    """RMSNorm over the last dimension with the rounding points of the modules behind
+    `attn.norm_q` / `attn.norm_k` (transformer_flux.py:120-121): diffusers' RMSNorm.forward
+    (diffusers>=0.33.0, models/normalization.py — a dependency that is not in the reference tree;
+    restated from its published source) and, with the same roundings, the in-tree
+    xfuser/model_executor/models/customized/step_video_t2v/normalization.py:34-60:
+        variance = x.float().pow(2).mean(-1) ; h = x * rsqrt(variance + eps)      (fp32)
+        16-bit weight: h = h.to(weight.dtype) * weight ; no weight: h.to(x.dtype)."""
+    input_dtype = x.dtype
+    variance = x.to(torch.float32).pow(2).mean(-1, keepdim=True)
+    h = x * torch.rsqrt(variance + eps)
+    if weight is not None:
+        if weight.dtype in (torch.float16, torch.bfloat16):
+            h = h.to(weight.dtype)
+        h = h * weight
+    else:
+        h = h.to(input_dtype)
+    return h
+
+
+def apply_rotary_emb_ref(x, freqs_cis, use_real_unbind_dim=-1, sequence_dim=2):
+    """diffusers' apply_rotary_emb with use_real=True (models/embeddings.py of diffusers>=0.33.0,
+    restated; called at transformer_flux.py:146-147 with sequence_dim=1 and at
+    transformer_hunyuan_video.py:60-83 with the default 2).  x [B,H,S,D] or [B,S,H,D];
+    freqs_cis = (cos, sin), each [S,D]."""
+    cos, sin = freqs_cis
+    if sequence_dim == 2:
+        cos, sin = cos[None, None, :, :], sin[None, None, :, :]
+    elif sequence_dim == 1:
+        cos, sin = cos[None, :, None, :], sin[None, :, None, :]
+    else:
+        raise ValueError(sequence_dim)
+    if use_real_unbind_dim == -1:
+        x_real, x_imag = x.reshape(*x.shape[:-1], -1, 2).unbind(-1)
+        x_rotated = torch.stack([-x_imag, x_real], dim=-1).flatten(3)
+    elif use_real_unbind_dim == -2:
+        x_real, x_imag = x.reshape(*x.shape[:-1], 2, -1).unbind(-2)
+        x_rotated = torch.cat([-x_imag, x_real], dim=-1)
+    else:
+        raise ValueError(use_real_unbind_dim)
+    return (x.float() * cos + x_rotated.float() * sin).to(x.dtype)
+
+
+def apply_rotary_emb_wan_ref(hidden_states, freqs_cos, freqs_sin):
+    """The local function of transformer_wan.py:108-120 ([B,S,H,D] input, [1,S,1,D] tables)."""
+    x1, x2 = hidden_states.unflatten(-1, (-1, 2)).unbind(-1)
+    cos = freqs_cos[..., 0::2]
+    sin = freqs_sin[..., 1::2]
+    out = torch.empty_like(hidden_states)
+    out[..., 0::2] = x1 * cos - x2 * sin
+    out[..., 1::2] = x1 * sin + x2 * cos
+    return out.type_as(hidden_states)
+
+
+def rope_tables(S, D, seed=0, axes=(16, 56, 56), theta=10000.0, interleave=True):
+    """Synthetic (cos, sin) tables [S, D] fp32 of the shape the DiT position embedders produce:
+    per axis a of width d_a, angle = pos_a * theta^(-2i/d_a); each angle repeated for the two
+    elements of its pair (`interleave`, the use_real_unbind_dim=-1 convention) or the table
+    repeated for the two halves (-2).  Positions are random integers per token and axis."""
+    g = torch.Generator().manual_seed(seed)
+    assert sum(axes) == D or axes == ()
+    if not axes:
+        axes = (D,)
+    cols = []
+    for d_a in axes:
+        pos = torch.randint(0, 64, (S,), generator=g).to(torch.float64)
+        freqs = 1.0 / (theta ** (torch.arange(0, d_a, 2, dtype=torch.float64) / d_a))
+        cols.append(torch.outer(pos, freqs))
+    ang = torch.cat(cols, dim=1)  # [S, D/2]
+    if interleave:
+        ang = ang.repeat_interleave(2, dim=1)
+    else:
+        ang = torch.cat([ang, ang], dim=1)
+    return ang.cos().float(), ang.sin().float()
 
 
 # ----------------------------------------------------------------------------------------------

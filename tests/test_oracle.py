@@ -280,3 +280,64 @@ def test_hadamard_rotate_ref_against_fwht_and_invariance(block):
     ye = O.hadamard_rotate_ref(e, block)
     assert torch.allclose(ye[..., :block].abs(), torch.full((block,), 64.0 * r, dtype=torch.float64))
     assert (ye[..., block:] == 0).all() or block == 128
+
+
+# ---------------------------------------------------------------------------- prologue
+def test_rms_norm_ref_against_torch_rms_norm_and_roundings():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2, 7, 3, 128, generator=g) * 3
+    w = 0.8 + 0.4 * torch.rand(128, generator=g)
+    # float64 inputs: no rounding anywhere except the fp32 statistic -> torch's own rms_norm
+    ref = F.rms_norm(x.double(), (128,), w.double(), 1e-6)
+    got = O.rms_norm_ref(x.double(), w.double(), 1e-6)
+    assert torch.allclose(got, ref, rtol=1e-6, atol=1e-7)
+    # a dropped eps or a mean over the wrong axis fails this
+    tiny = torch.full((1, 1, 1, 128), 1e-4)
+    assert torch.allclose(O.rms_norm_ref(tiny, None, 1e-6), tiny / (1e-8 + 1e-6) ** 0.5, rtol=1e-5)
+    # bf16: result = bf16(bf16(x * rs) * w), i.e. two roundings, and never further than 2 ulp from exact
+    xb, wb = x.bfloat16(), w.bfloat16()
+    got = O.rms_norm_ref(xb, wb, 1e-6)
+    assert got.dtype == torch.bfloat16
+    rs = torch.rsqrt(xb.float().pow(2).mean(-1, keepdim=True) + 1e-6)
+    two = ((xb.float() * rs).bfloat16().float() * wb.float()).bfloat16()
+    assert torch.equal(got, two)
+    exact = F.rms_norm(xb.double(), (128,), wb.double(), 1e-6)
+    assert ((got.double() - exact).abs() <= 2.0 ** -7 * exact.abs() + 1e-30).all()
+    assert O.rms_norm_ref(xb, None, 1e-6).dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("sequence_dim", [1, 2])
+def test_apply_rotary_emb_ref_is_complex_multiplication(sequence_dim):
+    g = torch.Generator().manual_seed(6)
+    S, D = 9, 16
+    x = torch.randn(2, 3, S, D, generator=g, dtype=torch.float64)
+    ang = torch.randn(S, D // 2, generator=g, dtype=torch.float64)
+    xin = x if sequence_dim == 2 else x.transpose(1, 2)
+    # interleaved pairs (2i, 2i+1) as complex numbers times e^{i angle}
+    cos, sin = ang.cos().repeat_interleave(2, 1), ang.sin().repeat_interleave(2, 1)
+    got = O.apply_rotary_emb_ref(xin, (cos, sin), -1, sequence_dim)
+    got = got if sequence_dim == 2 else got.transpose(1, 2)
+    z = torch.view_as_complex(x.reshape(2, 3, S, D // 2, 2).contiguous()) * torch.polar(torch.ones_like(ang), ang)
+    assert torch.allclose(got, torch.view_as_real(z).flatten(3), atol=1e-12)
+    # pairs (j, j + D/2)
+    cos2, sin2 = torch.cat([ang.cos()] * 2, 1), torch.cat([ang.sin()] * 2, 1)
+    got2 = O.apply_rotary_emb_ref(xin, (cos2, sin2), -2, sequence_dim)
+    got2 = got2 if sequence_dim == 2 else got2.transpose(1, 2)
+    z2 = torch.complex(x[..., :D // 2], x[..., D // 2:]) * torch.polar(torch.ones_like(ang), ang)
+    assert torch.allclose(got2, torch.cat([z2.real, z2.imag], -1), atol=1e-12)
+    # a rotation preserves the length of every pair; angle 0 is the identity
+    assert torch.allclose(got.reshape(2, 3, S, -1, 2).norm(dim=-1), x.reshape(2, 3, S, -1, 2).norm(dim=-1), atol=1e-12)
+    one, zero = torch.ones(S, D, dtype=torch.float64), torch.zeros(S, D, dtype=torch.float64)
+    assert torch.equal(O.apply_rotary_emb_ref(xin.float(), (one.float(), zero.float()), -1, sequence_dim), xin.float())
+    # the Wan form reads cos[2i] and sin[2i+1] for a pair: same result on pair-repeated tables
+    wan = O.apply_rotary_emb_wan_ref(x.transpose(1, 2), cos[None, :, None, :], sin[None, :, None, :])
+    assert torch.allclose(wan.transpose(1, 2), got, atol=1e-12)
+
+
+def test_rope_tables_shape_and_pairing():
+    cos, sin = O.rope_tables(11, 128, seed=1)
+    assert cos.shape == (11, 128) and cos.dtype == torch.float32
+    assert torch.equal(cos[:, 0::2], cos[:, 1::2]) and torch.equal(sin[:, 0::2], sin[:, 1::2])
+    assert torch.allclose(cos * cos + sin * sin, torch.ones(11, 128), atol=1e-6)
+    cos, sin = O.rope_tables(11, 64, seed=1, axes=(), interleave=False)
+    assert torch.equal(cos[:, :32], cos[:, 32:])

@@ -110,7 +110,35 @@ class QuantArgs(ctypes.Structure):
     ]
 
 
-EXPORTS = ("xdit_attn_fwd", "xdit_attn_workspace_bytes", "xdit_lse_merge", "xdit_fp8_quant", "xdit_attn_last_error", "xdit_attn_abi_version")
+class PrologueArgs(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32),
+        ("norm", ctypes.c_int32),
+        ("rope", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("eps", ctypes.c_float),
+        ("S", ctypes.c_int64),
+        ("x", ctypes.c_void_p),
+        ("y", ctypes.c_void_p),
+        ("weight", ctypes.c_void_p),
+        ("cos", ctypes.c_void_p),
+        ("sin", ctypes.c_void_p),
+        ("rope_stride", ctypes.c_int64),
+        ("rope_row0", ctypes.c_int64),
+        ("rope_rows", ctypes.c_int64),
+        ("x_stride", Strides),
+        ("y_stride", Strides),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+NORM_NONE, NORM_HEAD, NORM_TOKEN = 0, 1, 2
+ROPE_NONE, ROPE_INTERLEAVED, ROPE_SPLIT_HALF, ROPE_WAN = 0, 1, 2, 3
+
+EXPORTS = ("xdit_attn_fwd", "xdit_attn_workspace_bytes", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_attn_last_error", "xdit_attn_abi_version")
 
 _lib = None
 _lock = threading.Lock()
@@ -138,6 +166,8 @@ def lib():
         L.xdit_lse_merge.restype = ctypes.c_int
         L.xdit_fp8_quant.argtypes = [ctypes.POINTER(QuantArgs)]
         L.xdit_fp8_quant.restype = ctypes.c_int
+        L.xdit_qk_prologue.argtypes = [ctypes.POINTER(PrologueArgs)]
+        L.xdit_qk_prologue.restype = ctypes.c_int
         L.xdit_attn_last_error.argtypes = []
         L.xdit_attn_last_error.restype = ctypes.c_char_p
         L.xdit_attn_abi_version.argtypes = []

@@ -40,6 +40,25 @@ struct QuantParams {
   float had_scale;  // 1/sqrt(had_block) in fp32; the kernel rounds it to the input dtype
 };
 
+// Parameters of one prologue launch (RMSNorm + rotary embedding + re-layout of Q or K).
+struct PrologueParams {
+  const void* x;
+  void* y;
+  const void* weight;  // gain in the tensor's dtype: D entries (norm 1) or H*D (norm 2); may be null
+  const float* cos;
+  const float* sin;
+  int64_t xs_b, xs_h, xs_s;
+  int64_t ys_b, ys_h, ys_s;
+  int64_t rope_stride;  // elements between rows of cos / sin
+  int64_t rows;         // B * S * H
+  int B, H, S, D;
+  int norm;             // 0 none, 1 over head_dim per head, 2 over all heads of a token
+  int rope_mode;        // 0 none, 1 interleaved pairs, 2 split halves, 3 interleaved pairs, Wan's table indexing
+  int rope_row0, rope_rows;  // rows [row0, row0 + rows) of S are rotated, with table row s - row0
+  int lpr;              // lanes per row: smallest power of two >= D/8
+  float eps, inv_n;     // inv_n = 1 / number of elements under one norm statistic
+};
+
 // dtype codes below are the C ABI's xdit_dtype values: 0 bf16, 1 fp16, 2 fp32, 3 fp8 e4m3fn.
 hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream);
 size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block);
@@ -47,6 +66,8 @@ hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_pe
 size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block);
 hipError_t launch_attn_fwd_f32(const AttnParams& p, int dtype, int D, hipStream_t stream);
 hipError_t launch_fp8_quant(const QuantParams& p, int in_dtype, hipStream_t stream);
+hipError_t launch_qk_prologue(const PrologueParams& p, int dtype, hipStream_t stream);
+int prologue_max_token_elems();
 hipError_t launch_lse_merge(const MergeParams& p, int block_dtype, int final_dtype, hipStream_t stream);
 
 }  // namespace xdit

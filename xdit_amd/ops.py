@@ -200,3 +200,70 @@ def fp8_quant(x, per_tensor=False, scale=None, hadamard_block=0):
     with torch.cuda.device(device):
         _lib.check(_lib.lib().xdit_fp8_quant(ctypes.byref(a)))
     return y, descale
+
+
+_NORM_MODES = {None: _lib.NORM_NONE, "none": _lib.NORM_NONE, "head": _lib.NORM_HEAD, "token": _lib.NORM_TOKEN}
+_ROPE_MODES = {"interleaved": _lib.ROPE_INTERLEAVED, "split_half": _lib.ROPE_SPLIT_HALF, "wan": _lib.ROPE_WAN}
+
+
+def qk_prologue(x, weight=None, eps=1e-6, norm=None, rotary_emb=None, rope="interleaved",
+                rope_row0=0, rope_rows=None, out=None):
+    """RMSNorm + rotary embedding + re-layout of a logical BHSD tensor in one pass -> `out`
+    (logical BHSD, any strides; a new BHSD-contiguous tensor when omitted).
+
+    `norm`: None, "head" (over head_dim, `weight` has D entries) or "token" (over all heads of a
+    token, `weight` has H*D entries); `weight` is in x's dtype or None.  `rotary_emb` = (cos, sin),
+    fp32 tensors whose last dimension is D and whose rows (all other dimensions flattened) are the
+    positions; rows [rope_row0, rope_row0 + rope_rows) of S are rotated with table row s - rope_row0.
+    """
+    device = x.device
+    _check4("x", x, device)
+    B, H, S, D = x.shape
+    if out is None:
+        out = torch.empty((B, H, S, D), dtype=x.dtype, device=device)
+    else:
+        _check4("out", out, device)
+        if tuple(out.shape) != (B, H, S, D) or out.dtype != x.dtype:
+            raise ValueError("out has the wrong shape or dtype")
+    if norm not in _NORM_MODES:
+        raise ValueError("norm must be None, 'head' or 'token'")
+    a = _lib.PrologueArgs()
+    a.struct_size = ctypes.sizeof(_lib.PrologueArgs)
+    a.dtype = _code(x.dtype)
+    a.norm = _NORM_MODES[norm]
+    a.B, a.H, a.D, a.S = B, H, D, S
+    a.eps = float(eps)
+    a.x, a.y = x.data_ptr(), out.data_ptr()
+    a.x_stride, a.y_stride = _strides(x), _strides(out)
+    keep = []
+    if weight is not None and a.norm != _lib.NORM_NONE:
+        n = D if a.norm == _lib.NORM_HEAD else H * D
+        if weight.dtype != x.dtype or weight.numel() != n or weight.device != device:
+            raise ValueError("weight must have %d entries of dtype %s on %s" % (n, x.dtype, device))
+        weight = weight.reshape(-1).contiguous()
+        keep.append(weight)
+        a.weight = weight.data_ptr()
+    if rotary_emb is not None:
+        if rope not in _ROPE_MODES:
+            raise ValueError("rope must be one of %s" % (sorted(_ROPE_MODES),))
+        cos, sin = rotary_emb
+        for name, t in (("cos", cos), ("sin", sin)):
+            if t.dtype != torch.float32 or t.shape[-1] != D or t.device != device:
+                raise ValueError("%s must be an fp32 tensor with a last dimension of %d on %s" % (name, D, device))
+        cos = cos.reshape(-1, D)
+        sin = sin.reshape(-1, D)
+        if cos.stride(-1) != 1 or sin.stride(-1) != 1 or cos.stride(0) != sin.stride(0):
+            cos, sin = cos.contiguous(), sin.contiguous()
+        keep += [cos, sin]
+        if rope_rows is None:
+            rope_rows = min(cos.shape[0], S - rope_row0)
+        if cos.shape[0] < rope_rows or sin.shape[0] < rope_rows:
+            raise ValueError("the cos / sin tables hold %d rows, %d are needed" % (cos.shape[0], rope_rows))
+        a.rope = _ROPE_MODES[rope]
+        a.cos, a.sin = cos.data_ptr(), sin.data_ptr()
+        a.rope_stride = cos.stride(0)
+        a.rope_row0, a.rope_rows = int(rope_row0), int(rope_rows)
+    a.stream = _stream(device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().xdit_qk_prologue(ctypes.byref(a)))
+    return out
