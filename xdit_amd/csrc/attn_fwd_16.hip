@@ -15,16 +15,21 @@
 // and the S^T accumulator registers are, after conversion to 16 bit, exactly the B operand of
 // the second product, so P never goes through LDS.
 //
-// LDS layout: see attn_tiles.h.  The workgroup has NW = 4 or 8 wavefronts (128 or 256 query rows):
-// 8 wavefronts share every K/V tile, which halves the L2->LDS traffic per FLOP, and are used
-// when the problem still yields enough workgroups to fill the chip.
+// LDS layout: see attn_tiles.h.  The workgroup has NW = 4, 8 or 12 wavefronts (128 / 256 / 384
+// query rows): 8 or 12 wavefronts share every K/V tile, which cuts the L2->LDS traffic per FLOP
+// to a half or a third, and are used when the problem still yields enough workgroups to fill
+// the chip.
+//
+// LDS fragment reads are issued by hand (inline assembly, kPrefetch MFMAs ahead of their use,
+// completion awaited with counted s_waitcnt): left to the compiler, every MFMA waits for a read
+// issued just before it, and the read latency is paid sixteen times per product and tile.
 #include "attn_split.h"
 #include "launchers.h"
 
 namespace xdit {
 
 constexpr int kRowsPerWave = 32;
-// K fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
+// LDS fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
 constexpr int kPrefetch = 4;
 
 // One segment of work: the query tile `tile`, KV tiles [it0, it1).  With `part_out == nullptr` the
@@ -72,46 +77,59 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   const T* kbase2 = p.Sk2 > 0 ? (const T*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
   const T* vbase2 = p.Sk2 > 0 ? (const T*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
   constexpr int LANES_PER_ROW = G::ROW_BYTES / 16;
-  constexpr int PIECES = 2 * G::NG;
-  constexpr int LOADS = (PIECES + kWaves - 1) / kWaves;  // pieces per wavefront per tile
-  const int ld_row0 = G::NG * (lane / LANES_PER_ROW);       // row of this lane's slot within piece 0
-  const unsigned ld_colb = (lane % LANES_PER_ROW) * 16;     // byte offset inside the row
+  // Loader wavefronts: the first LW wavefronts each load PAIRS (K piece g, V piece g) pairs,
+  // g = wave + LW * i, with one row index per lane for both pieces of a pair.
+  constexpr int LW = kWaves < 8 ? kWaves : 8;
+  constexpr int PAIRS = G::NG / LW;
+  static_assert(G::NG % LW == 0, "pieces must divide evenly over the loader wavefronts");
+  const int ld_row0 = G::NG * (lane / LANES_PER_ROW) + wave;  // row of this lane in pair 0
+  const unsigned ld_colb = (lane % LANES_PER_ROW) * 16;       // byte offset inside the row
   const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS unsigned char*)smem;
+  const unsigned ld_kdst = lds_base + wave * G::K_PITCH;      // LDS address of K piece `wave`, buffer 0
+  const unsigned ld_vdst = lds_base + G::K_BYTES + wave * G::V_PITCH;
 
   const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
   const int nt2 = (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
   const int nt = nt1 + nt2;
 
-  auto issue_tile = [&](int t, int buf) {
-    const unsigned kdst = lds_base + buf * G::BUF_BYTES;
-    const unsigned vdst = kdst + G::K_BYTES;
-    const T* kb;
-    const T* vb;
-    unsigned kss, vss;
-    int valid;
+  // Stream position: base pointers of the next tile to load, byte strides, keys left in its segment.
+  const T* ld_kp;
+  const T* ld_vp;
+  unsigned ld_kss, ld_vss;
+  int64_t ld_kstep, ld_vstep;
+  int ld_left;
+  auto seek_tile = [&](int t) {
     if (t < nt1) {
-      kb = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
-      vb = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
-      kss = (unsigned)(p.ks_s * 2); vss = (unsigned)(p.vs_s * 2);
-      valid = p.Sk - t * kKeysPerTile;
+      ld_kp = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
+      ld_vp = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
+      ld_kss = (unsigned)(p.ks_s * 2); ld_vss = (unsigned)(p.vs_s * 2);
+      ld_kstep = kKeysPerTile * p.ks_s; ld_vstep = kKeysPerTile * p.vs_s;
+      ld_left = p.Sk - t * kKeysPerTile;
     } else {
-      kb = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
-      vb = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
-      kss = (unsigned)(p.k2s_s * 2); vss = (unsigned)(p.v2s_s * 2);
-      valid = p.Sk2 - (t - nt1) * kKeysPerTile;
+      ld_kp = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
+      ld_vp = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
+      ld_kss = (unsigned)(p.k2s_s * 2); ld_vss = (unsigned)(p.v2s_s * 2);
+      ld_kstep = kKeysPerTile * p.k2s_s; ld_vstep = kKeysPerTile * p.v2s_s;
+      ld_left = p.Sk2 - (t - nt1) * kKeysPerTile;
     }
-    const int last = (valid < kKeysPerTile ? valid : kKeysPerTile) - 1;
+  };
+  // Loads the tile at the stream position into buffer `buf` and advances the position.
+  auto issue_tile = [&](int t, int buf) {
+    if (kWaves == LW || wave < LW) {
+      const int last = (ld_left < kKeysPerTile ? ld_left : kKeysPerTile) - 1;
+      const unsigned bo = buf * G::BUF_BYTES;
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) {
-      const int pi = wave + kWaves * i;  // wavefront-uniform
-      if (pi < PIECES) {
-        const bool is_v = pi >= G::NG;
-        const int g = is_v ? pi - G::NG : pi;
-        int r = g + ld_row0;
+      for (int i = 0; i < PAIRS; i++) {
+        int r = ld_row0 + LW * i;
         r = r < last ? r : last;  // rows past the end of the segment re-read its last row
-        if (is_v) load_lds_16(vb, __umul24((unsigned)r, vss) + ld_colb, vdst + g * G::V_PITCH);
-        else load_lds_16(kb, __umul24((unsigned)r, kss) + ld_colb, kdst + g * G::K_PITCH);
+        load_lds_16(ld_kp, __umul24((unsigned)r, ld_kss) + ld_colb, ld_kdst + bo + i * LW * G::K_PITCH);
+        load_lds_16(ld_vp, __umul24((unsigned)r, ld_vss) + ld_colb, ld_vdst + bo + i * LW * G::V_PITCH);
       }
+    }
+    if (t + 1 == nt1) {
+      seek_tile(t + 1);
+    } else {
+      ld_kp += ld_kstep; ld_vp += ld_vstep; ld_left -= kKeysPerTile;
     }
   };
 
@@ -141,6 +159,7 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
 
+  seek_tile(it0);
   issue_tile(it0, 0);
   // Make the compiler account for the Q fragment loads here, before the loop: the tile loads
   // above are invisible to its outstanding-load bookkeeping, so any wait it placed for a Q
@@ -163,17 +182,30 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
 
     // ---- S^T = K Q^T : 2 blocks of 32 keys x 32 queries ---------------------------------
     f32x16 sacc[2];
+    {
+      constexpr int PD = kPrefetch;   // K fragment reads in flight
+      constexpr int NR = 2 * KSTEPS;  // reads (= MFMAs) of this product
+      const unsigned kaddr = (unsigned)(uintptr_t)ktile;
+      vec8 kf[NR];
+      static_for<PD>([&](auto I) {
+        constexpr int i = I;
+        lds_read_b128<(i / KSTEPS) * K_KB_STEP + (i % KSTEPS) * 32>(kf[i], kaddr);
+      });
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
+      for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        vec8 kf = *(const XDIT_LDS vec8*)(ktile + kb * K_KB_STEP + ks * 32);
-        sacc[kb] = Mfma16<T>::mma(kf, qf[ks], sacc[kb]);
-      }
+        for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+      static_for<NR>([&](auto I) {
+        constexpr int i = I;
+        constexpr int younger = (i + PD <= NR ? PD : NR - i) - 1;
+        lds_wait<younger>(kf[i]);
+        sacc[i / KSTEPS] = Mfma16<T>::mma(kf[i], qf[i % KSTEPS], sacc[i / KSTEPS]);
+        if constexpr (i + PD < NR) {
+          constexpr int n = i + PD;
+          lds_read_b128<(n / KSTEPS) * K_KB_STEP + (n % KSTEPS) * 32>(kf[n], kaddr);
+        }
+      });
     }
-
     // ---- mask keys past the end of the segment (only its last tile can be partial) -------
     const int valid = (t < nt1) ? p.Sk - t * kKeysPerTile : p.Sk2 - (t - nt1) * kKeysPerTile;
     if (valid < kKeysPerTile) {
@@ -222,18 +254,31 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
     }
 
     // ---- O^T += V^T P^T ------------------------------------------------------------------
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-#pragma unroll
-      for (int db = 0; db < DBLOCKS; db++) {
-        typedef __attribute__((ext_vector_type(8))) short s16x8;
-        s16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (XDIT_LDS s16x4*)(vtile + j * V_J_STEP + db * 64));
-        s16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (XDIT_LDS s16x4*)(vtile + j * V_J_STEP + db * 64 + V_RD_STEP));
-        s16x8 vv = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
-        oacc[db] = Mfma16<T>::mma(__builtin_bit_cast(vec8, vv), pf[j], oacc[db]);
-      }
+    {
+      constexpr int PD = kPrefetch;  // MFMAs whose two V^T reads are in flight
+      constexpr int NM = 4 * DBLOCKS;
+      typedef __attribute__((ext_vector_type(8))) short s16x8;
+      const unsigned vaddr = (unsigned)(uintptr_t)vtile;
+      s16x4 v0[NM], v1[NM];
+      static_for<PD>([&](auto I) {
+        constexpr int i = I;
+        constexpr int off = (i / DBLOCKS) * V_J_STEP + (i % DBLOCKS) * 64;
+        lds_read_tr16_b64<off>(v0[i], vaddr);
+        lds_read_tr16_b64<off + V_RD_STEP>(v1[i], vaddr);
+      });
+      static_for<NM>([&](auto I) {
+        constexpr int i = I;
+        constexpr int younger = 2 * ((i + PD <= NM ? PD : NM - i) - 1);
+        lds_wait2<younger>(v0[i], v1[i]);
+        s16x8 vv = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        oacc[i % DBLOCKS] = Mfma16<T>::mma(__builtin_bit_cast(vec8, vv), pf[i / DBLOCKS], oacc[i % DBLOCKS]);
+        if constexpr (i + PD < NM) {
+          constexpr int n = i + PD;
+          constexpr int off = (n / DBLOCKS) * V_J_STEP + (n % DBLOCKS) * 64;
+          lds_read_tr16_b64<off>(v0[n], vaddr);
+          lds_read_tr16_b64<off + V_RD_STEP>(v1[n], vaddr);
+        }
+      });
     }
   }
 

@@ -1,6 +1,8 @@
 // Pieces shared by the 16-bit attention kernels: MFMA wrappers, the LDS tile geometry and the
 // direct global->LDS load.
 #pragma once
+#include <utility>
+
 #include "common.h"
 
 namespace xdit {
@@ -58,6 +60,37 @@ __device__ __forceinline__ void load_lds_16(const void* base, unsigned off, unsi
       :
       : "s"(lds), "v"(off), "s"(base)
       : "memory", "m0");
+}
+
+// Compile-time loop: f(std::integral_constant<int, I>) for I = 0..N-1.
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+// LDS reads issued by hand so that several are in flight.  The compiler does not know that the
+// destination is still in flight, so before its first use it must go through lds_wait<N>(x) (or
+// lds_wait2 for two registers): N is the number of LDS reads issued AFTER the one being awaited;
+// LDS returns data in order, so "at most N outstanding" means that read has landed.  Reads the
+// compiler issues in between only make the wait stricter.
+template <int OFF, typename V>
+__device__ __forceinline__ void lds_read_b128(V& dst, unsigned addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int OFF, typename V>
+__device__ __forceinline__ void lds_read_tr16_b64(V& dst, unsigned addr) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int N, typename V>
+__device__ __forceinline__ void lds_wait(V& x) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
+}
+template <int N, typename V>
+__device__ __forceinline__ void lds_wait2(V& x, V& y) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
 }
 
 }  // namespace xdit
