@@ -1,9 +1,9 @@
 // Non-causal attention forward for fp8 (OCP e4m3fn) Q/K/V with per-(batch, head) fp32 descales,
 // head_dim 128, bf16 or fp16 output, fp32 log-sum-exp, on gfx950.
 //
-// Same structure as the 16-bit kernel (workgroup = 4 wavefronts x 32 query rows, 64-key K/V
-// tiles double buffered in LDS by direct global->LDS loads, transposed products so that each lane
-// owns one query), with v_mfma_f32_32x32x64_f8f6f4 for both products:
+// Same structure as the 16-bit kernel (workgroup = 4, 8 or 12 wavefronts x 32 query rows, 64-key
+// K/V tiles double buffered in LDS by direct global->LDS loads, hand-issued LDS fragment reads,
+// transposed products so that each lane owns one query), with v_mfma_f32_32x32x64_f8f6f4 for both products:
 //   S^T = K Q^T    A = K rows, B = Q^T (registers); contraction over head_dim, 64 per instruction.
 //                  A and B use the same lane->contraction-index map, so each lane simply holds the
 //                  32 contiguous bytes d = 64ks + 32(l/32) .. +31 of its row.
@@ -38,7 +38,8 @@ constexpr int V_PITCH = 1024 + 32;
 constexpr int K_BYTES = NG * K_PITCH;
 constexpr int V_BYTES = NG * V_PITCH;
 constexpr int BUF_BYTES = K_BYTES + V_BYTES;
-constexpr int PIECES = 2 * NG;  // 1 KiB pieces per tile: K pieces 0..NG-1, then V pieces
+// LDS fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
+constexpr int kPrefetch = 2;
 
 // One segment of work: query tile `tile`, KV tiles [it0, it1); see attn_split.h for part_out.
 template <typename TO, int NW>
@@ -47,7 +48,6 @@ __device__ __forceinline__ void attn_segment_fp8(const AttnParams& p, unsigned c
   typedef unsigned char u8;
   constexpr int kWaves = NW;
   constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
-  constexpr int LOADS = (PIECES + kWaves - 1) / kWaves;  // pieces per wavefront per tile
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -77,41 +77,55 @@ __device__ __forceinline__ void attn_segment_fp8(const AttnParams& p, unsigned c
   const u8* vbase1 = (const u8*)p.v + b * p.vs_b + h * p.vs_h;
   const u8* kbase2 = p.Sk2 > 0 ? (const u8*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
   const u8* vbase2 = p.Sk2 > 0 ? (const u8*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
-  const int ld_row0 = NG * (lane >> 3);           // 8 lanes per 128-byte row: row of this lane's slot in piece 0
+  // Loader wavefronts: the first LW wavefronts each load PAIRS (K piece g, V piece g) pairs,
+  // g = wave + LW * i, with one row index per lane for both pieces of a pair.
+  constexpr int LW = kWaves < 8 ? kWaves : 8;
+  constexpr int PAIRS = NG / LW;
+  const int ld_row0 = NG * (lane >> 3) + wave;    // 8 lanes per 128-byte row: row of this lane in pair 0
   const unsigned ld_colb = (lane & 7) * 16;
   const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS u8*)smem;
+  const unsigned ld_kdst = lds_base + wave * K_PITCH;  // LDS address of K piece `wave`, buffer 0
+  const unsigned ld_vdst = lds_base + K_BYTES + wave * V_PITCH;
   const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
 
-  auto issue_tile = [&](int t, int buf) {
-    const unsigned kdst = lds_base + buf * BUF_BYTES;
-    const unsigned vdst = kdst + K_BYTES;
-    const u8* kb;
-    const u8* vb;
-    unsigned kss, vss;
-    int valid;
+  // Stream position: base pointers of the next tile to load, byte strides, keys left in its segment.
+  const u8* ld_kp;
+  const u8* ld_vp;
+  unsigned ld_kss, ld_vss;
+  int64_t ld_kstep, ld_vstep;
+  int ld_left;
+  auto seek_tile = [&](int t) {
     if (t < nt1) {
-      kb = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
-      vb = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
-      kss = (unsigned)p.ks_s; vss = (unsigned)p.vs_s;
-      valid = p.Sk - t * kKeysPerTile;
+      ld_kp = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
+      ld_vp = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
+      ld_kss = (unsigned)p.ks_s; ld_vss = (unsigned)p.vs_s;
+      ld_kstep = kKeysPerTile * p.ks_s; ld_vstep = kKeysPerTile * p.vs_s;
+      ld_left = p.Sk - t * kKeysPerTile;
     } else {
-      kb = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
-      vb = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
-      kss = (unsigned)p.k2s_s; vss = (unsigned)p.v2s_s;
-      valid = p.Sk2 - (t - nt1) * kKeysPerTile;
+      ld_kp = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
+      ld_vp = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
+      ld_kss = (unsigned)p.k2s_s; ld_vss = (unsigned)p.v2s_s;
+      ld_kstep = kKeysPerTile * p.k2s_s; ld_vstep = kKeysPerTile * p.v2s_s;
+      ld_left = p.Sk2 - (t - nt1) * kKeysPerTile;
     }
-    const int last = (valid < kKeysPerTile ? valid : kKeysPerTile) - 1;
+  };
+  // Loads the tile at the stream position into buffer `buf` and advances the position.
+  auto issue_tile = [&](int t, int buf) {
+    if (kWaves == LW || wave < LW) {
+      const int last = (ld_left < kKeysPerTile ? ld_left : kKeysPerTile) - 1;
+      const unsigned bo = buf * BUF_BYTES;
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) {
-      const int pi = wave + kWaves * i;  // wavefront-uniform
-      if (pi < PIECES) {
-        const bool is_v = pi >= NG;
-        const int g = is_v ? pi - NG : pi;
-        int r = g + ld_row0;
+      for (int i = 0; i < PAIRS; i++) {
+        int r = ld_row0 + LW * i;
         r = r < last ? r : last;  // rows past the end of the segment re-read its last row
-        if (is_v) load_lds_16(vb, __umul24((unsigned)r, vss) + ld_colb, vdst + g * V_PITCH);
-        else load_lds_16(kb, __umul24((unsigned)r, kss) + ld_colb, kdst + g * K_PITCH);
+        load_lds_16(ld_kp, __umul24((unsigned)r, ld_kss) + ld_colb, ld_kdst + bo + i * LW * K_PITCH);
+        load_lds_16(ld_vp, __umul24((unsigned)r, ld_vss) + ld_colb, ld_vdst + bo + i * LW * V_PITCH);
       }
+    }
+    if (t + 1 == nt1) {
+      seek_tile(t + 1);
+    } else {
+      ld_kp += ld_kstep; ld_vp += ld_vstep; ld_left -= kKeysPerTile;
     }
   };
 
@@ -140,6 +154,7 @@ __device__ __forceinline__ void attn_segment_fp8(const AttnParams& p, unsigned c
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
 
+  seek_tile(it0);
   issue_tile(it0, 0);
 #pragma unroll
   for (int ks = 0; ks < 2; ks++) asm volatile("" : "+v"(qf[ks]));
@@ -154,18 +169,36 @@ __device__ __forceinline__ void attn_segment_fp8(const AttnParams& p, unsigned c
     const XDIT_LDS u8* vtile = (const XDIT_LDS u8*)(smem + buf * BUF_BYTES + K_BYTES) + vbase_off;
 
     // ---- S^T = K Q^T ---------------------------------------------------------------------
+    // Four MFMAs; MFMA m = 2 kb + ks takes the 32 bytes of its K row as two 16-byte reads.
     f32x16 sacc[2];
+    {
+      constexpr int PD = kPrefetch;  // MFMAs whose two reads are in flight
+      constexpr int NM = 4;
+      const unsigned kaddr = (unsigned)(uintptr_t)ktile;
+      i32x4 klo[NM], khi[NM];
+      static_for<PD>([&](auto I) {
+        constexpr int m = I;
+        constexpr int off = (m / 2) * 4 * ROW_BYTES + (m % 2) * 64;
+        lds_read_b128<off>(klo[m], kaddr);
+        lds_read_b128<off + 16>(khi[m], kaddr);
+      });
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
+      for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-        i32x4 lo = *(const XDIT_LDS i32x4*)(ktile + kb * 4 * ROW_BYTES + ks * 64);
-        i32x4 hi = *(const XDIT_LDS i32x4*)(ktile + kb * 4 * ROW_BYTES + ks * 64 + 16);
-        i32x8 kf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[ks], sacc[kb], 0, 0, 0, 0, 0, 0);
-      }
+        for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+      static_for<NM>([&](auto I) {
+        constexpr int m = I;
+        constexpr int younger = 2 * ((m + PD <= NM ? PD : NM - m) - 1);
+        lds_wait2<younger>(klo[m], khi[m]);
+        i32x8 kf = __builtin_shufflevector(klo[m], khi[m], 0, 1, 2, 3, 4, 5, 6, 7);
+        sacc[m / 2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[m % 2], sacc[m / 2], 0, 0, 0, 0, 0, 0);
+        if constexpr (m + PD < NM) {
+          constexpr int n = m + PD;
+          constexpr int off = (n / 2) * 4 * ROW_BYTES + (n % 2) * 64;
+          lds_read_b128<off>(klo[n], kaddr);
+          lds_read_b128<off + 16>(khi[n], kaddr);
+        }
+      });
     }
 
     const int valid = (t < nt1) ? p.Sk - t * kKeysPerTile : p.Sk2 - (t - nt1) * kKeysPerTile;
@@ -215,16 +248,38 @@ __device__ __forceinline__ void attn_segment_fp8(const AttnParams& p, unsigned c
     }
 
     // ---- O^T += V^T P^T ------------------------------------------------------------------
+    // Four MFMAs (d blocks); each takes its V^T operand as four transposing 8-byte reads.
+    {
+      constexpr int PD = kPrefetch;
+      constexpr int NM = 4;
+      const unsigned vaddr = (unsigned)(uintptr_t)vtile;
+      i32x2 vr[NM][4];
+      static_for<PD>([&](auto I) {
+        constexpr int m = I;
+        static_for<4>([&](auto R) {
+          constexpr int r = R;
+          lds_read_tr8_b64<r * 2 * ROW_BYTES + m * 32>(vr[m][r], vaddr);
+        });
+      });
+      static_for<NM>([&](auto I) {
+        constexpr int m = I;
+        constexpr int younger = 4 * ((m + PD <= NM ? PD : NM - m) - 1);
+        lds_wait4<younger>(vr[m][0], vr[m][1], vr[m][2], vr[m][3]);
+        i32x8 vf;
 #pragma unroll
-    for (int db = 0; db < 4; db++) {
-      i32x8 vf;
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        i32x2 x = __builtin_amdgcn_ds_read_tr8_b64_v2i32((XDIT_LDS i32x2*)(vtile + r * 2 * ROW_BYTES + db * 32));
-        vf[2 * r] = x[0];
-        vf[2 * r + 1] = x[1];
-      }
-      oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[db], 0, 0, 0, 0, 0, 0);
+        for (int r = 0; r < 4; r++) {
+          vf[2 * r] = vr[m][r][0];
+          vf[2 * r + 1] = vr[m][r][1];
+        }
+        oacc[m] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[m], 0, 0, 0, 0, 0, 0);
+        if constexpr (m + PD < NM) {
+          constexpr int n = m + PD;
+          static_for<4>([&](auto R) {
+            constexpr int r = R;
+            lds_read_tr8_b64<r * 2 * ROW_BYTES + n * 32>(vr[n][r], vaddr);
+          });
+        }
+      });
     }
   }
 

@@ -84,6 +84,10 @@ template <int OFF, typename V>
 __device__ __forceinline__ void lds_read_tr16_b64(V& dst, unsigned addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
 }
+template <int OFF, typename V>
+__device__ __forceinline__ void lds_read_tr8_b64(V& dst, unsigned addr) {
+  asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
 template <int N, typename V>
 __device__ __forceinline__ void lds_wait(V& x) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
@@ -91,6 +95,11 @@ __device__ __forceinline__ void lds_wait(V& x) {
 template <int N, typename V>
 __device__ __forceinline__ void lds_wait2(V& x, V& y) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+}
+
+template <int N, typename V>
+__device__ __forceinline__ void lds_wait4(V& x, V& y, V& z, V& w) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x), "+v"(y), "+v"(z), "+v"(w) : "n"(N));
 }
 
 }  // namespace xdit
