@@ -212,7 +212,7 @@ int xdit_fp8_quant(const xdit_quant_args* a) {
   if (a->B <= 0 || a->H <= 0 || a->S <= 0) return fail(XDIT_ERR_INVALID_ARG, "B, H, S must be positive");
   if (a->B * (int64_t)a->H > 65535) return fail(XDIT_ERR_INVALID_ARG, "B*H above 65535");
   if (a->per_tensor && a->B * (int64_t)a->H > 1024) return fail(XDIT_ERR_INVALID_ARG, "per_tensor mode supports B*H <= 1024");
-  if (a->D <= 0 || a->D % 8 != 0) return fail(XDIT_ERR_INVALID_ARG, "head_dim %d must be a positive multiple of 8", a->D);
+  if (a->D <= 0 || a->D % 8 != 0 || a->D > 2048) return fail(XDIT_ERR_INVALID_ARG, "head_dim %d must be a positive multiple of 8, at most 2048", a->D);
   if (a->S > (int64_t(1) << 30)) return fail(XDIT_ERR_INVALID_ARG, "S above 2^30");
   if (a->descale == nullptr) return fail(XDIT_ERR_INVALID_ARG, "descale is NULL");
   int rc;

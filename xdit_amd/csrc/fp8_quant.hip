@@ -73,24 +73,50 @@ __global__ void fill_zero_kernel(float* p, int n) {
   if (i < n) p[i] = 0.f;
 }
 
-// grid = (blocks per slice, B*H); each thread walks 8-element chunks of its (b,h) slice.
+// Both tensor passes: grid = (blocks per slice, B*H).  A row of D elements is held by D/8
+// consecutive threads (8 elements each), a workgroup covers 256 / (D/8) rows per step and every
+// thread keeps kRowsInFlight rows in flight; rows advance by whole grid steps, so there is no
+// division in the loop and the trip count is the same for every thread of a workgroup (the
+// lanes of a row exchange data in the Hadamard rotation).
+constexpr int kRowsInFlight = 4;
+
+template <typename T, typename F>
+__device__ __forceinline__ void for_each_chunk(const QuantParams& p, const T* x, F&& f) {
+  const int cpr = p.D >> 3;
+  const int rpb = 256 / cpr;              // rows per workgroup step
+  const int c = threadIdx.x % cpr;
+  const int r = threadIdx.x / cpr;
+  const bool lane_live = r < rpb;
+  const int64_t step = (int64_t)gridDim.x * rpb;
+  for (int64_t base = (int64_t)blockIdx.x * rpb; base < p.S; base += step * kRowsInFlight) {
+    float v[kRowsInFlight][8];
+    int64_t s[kRowsInFlight];
+#pragma unroll
+    for (int j = 0; j < kRowsInFlight; j++) {
+      s[j] = base + j * step + r;
+      const int64_t sc = s[j] < p.S ? s[j] : p.S - 1;  // rows past the end re-read the last row
+      load8<T>(x + sc * p.xs_s + c * 8, v[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < kRowsInFlight; j++) {
+      if (p.had_block > 1) hadamard_rows<T>(v[j], p.had_block, p.had_scale, c);
+      f(v[j], s[j], c, lane_live && s[j] < p.S);
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void absmax_kernel(const QuantParams p) {
   const int bh = blockIdx.y;
   const int b = bh / p.H, h = bh - b * p.H;
   const T* x = (const T*)p.x + b * p.xs_b + h * p.xs_h;
-  const int cpr = p.D >> 3;
-  const int64_t chunks = (int64_t)p.S * cpr;
   float m = 0.f;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * 256) {
-    const int64_t s = i / cpr;
-    const int c = (int)(i - s * cpr);
-    float v[8];
-    load8<T>(x + s * p.xs_s + c * 8, v);
-    if (p.had_block > 1) hadamard_rows<T>(v, p.had_block, p.had_scale, c);
+  for_each_chunk<T>(p, x, [&](float (&v)[8], int64_t, int, bool live) {
+    if (live) {
 #pragma unroll
-    for (int j = 0; j < 8; j++) m = fmaxf(m, fabsf(v[j]));  // fmaxf drops NaN operands
-  }
+      for (int j = 0; j < 8; j++) m = fmaxf(m, fabsf(v[j]));  // fmaxf drops NaN operands
+    }
+  });
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
   __shared__ float wm[4];
@@ -116,14 +142,7 @@ __global__ __launch_bounds__(256) void cast_kernel(const QuantParams p) {
     const float am = p.amax[p.per_tensor ? 0 : bh];
     scale = am > 0.f ? am / kFp8Max : 1.0f;
   }
-  const int cpr = p.D >> 3;
-  const int64_t chunks = (int64_t)p.S * cpr;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * 256) {
-    const int64_t s = i / cpr;
-    const int c = (int)(i - s * cpr);
-    float v[8];
-    load8<T>(x + s * p.xs_s + c * 8, v);
-    if (p.had_block > 1) hadamard_rows<T>(v, p.had_block, p.had_scale, c);
+  for_each_chunk<T>(p, x, [&](float (&v)[8], int64_t s, int c, bool live) {
 #pragma unroll
     for (int j = 0; j < 8; j++) v[j] = v[j] / scale;
     int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
@@ -131,8 +150,8 @@ __global__ __launch_bounds__(256) void cast_kernel(const QuantParams p) {
     int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], 0, false);
     w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], w1, true);
     i32x2 w = {w0, w1};
-    *(i32x2*)(y + s * p.ys_s + c * 8) = w;
-  }
+    if (live) *(i32x2*)(y + s * p.ys_s + c * 8) = w;
+  });
 }
 
 // amax buffer -> descale values, for all B*H entries.
@@ -150,14 +169,19 @@ __global__ void finalize_kernel(const QuantParams p, int n) {
 template <typename T>
 static hipError_t run(const QuantParams& p, hipStream_t stream) {
   const int BH = p.B * p.H;
-  const int64_t chunks = (int64_t)p.S * (p.D >> 3);
-  int per_slice = (int)((chunks + 256 * 8 - 1) / (256 * 8));  // ~8 chunks per thread
+  const int rpb = 256 / (p.D >> 3);
+  int per_slice = (int)(((int64_t)p.S + rpb * 2 * quant::kRowsInFlight - 1) / (rpb * 2 * quant::kRowsInFlight));  // ~8 rows per thread
   if (per_slice < 1) per_slice = 1;
   if (per_slice > 2048) per_slice = 2048;
   dim3 grid(per_slice, BH), block(256);
   if (p.scale_in == nullptr) {
+    // every workgroup ends in one atomic max on its slice's entry: keep their number near 1024,
+    // same-address atomics are served one at a time
+    int reduce_slice = 1024 / BH;
+    if (reduce_slice < 1) reduce_slice = 1;
+    if (reduce_slice > per_slice) reduce_slice = per_slice;
     hipLaunchKernelGGL(fill_zero_kernel, dim3((BH + 255) / 256), dim3(256), 0, stream, p.amax, BH);
-    hipLaunchKernelGGL((absmax_kernel<T>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((absmax_kernel<T>), dim3(reduce_slice, BH), block, 0, stream, p);
   }
   hipLaunchKernelGGL((cast_kernel<T>), grid, block, 0, stream, p);
   // per_tensor broadcasts entry 0: keep it to one workgroup so the barrier orders read/write
