@@ -179,6 +179,19 @@ def main():
         fn = usp._get_attention_function()
         _, ms = time_calls(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), n, 3)
         also["c3_flux_ring4"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        # the same ring captured once in a HIP graph and replayed (shows whether the eager form is launch-bound)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            usp.ring_attn(fn, q, k, v, ring_chunks=4)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            usp.ring_attn(fn, q, k, v, ring_chunks=4)
+        _, ms = time_calls(graph.replay, n, 3)
+        also["c3_flux_ring4_graph"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        del graph
         # the merge kernel alone: bytes per fold = 10*N*D + 12*N
         N = B * H * S
         acc = torch.randn(B, H, S, D, device=dev)

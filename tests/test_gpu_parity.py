@@ -508,3 +508,35 @@ def test_custom_ops_opcheck_and_compile(gpu):
     e8 = fp8_block(q, k, v)
     c8 = torch.compile(fp8_block, backend="aot_eager", fullgraph=True)(q, k, v)
     assert torch.equal(c8[0], e8[0]) and torch.equal(c8[1], e8[1])
+
+
+# ---------------------------------------------------------------------------- HIP graphs
+def test_graph_capture_and_replay_of_the_ring(gpu):
+    """The launch-bound ring of four chunks (4 attention launches + combine + 4 merge launches)
+    captured once in a HIP graph and replayed: every replay must equal the eager result for the
+    inputs in the static buffers at that time, with eager launches and synchronisations between
+    the replays (the workspace and all temporaries live in the graph's memory pool)."""
+    fn = usp._get_attention_function()
+    q, k, v = O.make_qkv(1, 8, 1536, 128, seed=81, rmsnorm=True, dtype=torch.bfloat16)
+    sq, sk, sv = q.to(gpu), k.to(gpu), v.to(gpu)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):      # warm-up off the default stream, as graph capture requires
+        for _ in range(2):
+            usp.ring_attn(fn, sq, sk, sv, ring_chunks=4)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sout = usp.ring_attn(fn, sq, sk, sv, ring_chunks=4)
+    for seed in (82, 83, 84):
+        q2, k2, v2 = O.make_qkv(1, 8, 1536, 128, seed=seed, rmsnorm=True, dtype=torch.bfloat16)
+        sq.copy_(q2.to(gpu)); sk.copy_(k2.to(gpu)); sv.copy_(v2.to(gpu))
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = sout.clone()
+        eager = usp.ring_attn(fn, sq, sk, sv, ring_chunks=4)   # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, eager)
+        ro, _ = O.attn_fwd_ref(q2, k2, v2)
+        assert _err(replayed, ro) <= 2e-2
