@@ -8,7 +8,7 @@
 #include <cstdlib>
 #include <cstring>
 
-#include "common.h"
+#include "attn_split.h"
 #include "launchers.h"
 
 namespace {
@@ -52,8 +52,13 @@ int check_tensor(const char* name, const void* p, const xdit_strides& st, int es
   return 0;
 }
 
-// Query rows per workgroup for the 16-bit kernel: 384 (12 wavefronts sharing each K/V tile, 3 per
-// SIMD) or 256 (8) when that still yields enough workgroups to fill the 256 CUs, else 128.
+// Query rows per workgroup (head_dim 128: 384, 256 or 128, i.e. 12, 8 or 4 wavefronts sharing each
+// K/V tile).  Picks the shape with the shortest estimated critical path: KV iterations of the
+// busiest compute unit (whole rounds of resident workgroups, or the balanced launch's shared last
+// round plus its fixed cost) times the rows a compute unit works on per iteration, with a small
+// penalty for the shapes that share a tile between fewer wavefronts.  Measured on Flux-1024
+// (72 KV tiles: 384 rows wins through the balanced launch) and on its ring chunks (18 KV tiles:
+// 256 rows, 0.079 ms against 0.101 ms at 384).
 int rows_per_block_16(const xdit_attn_args* a) {
   if (a->D != 128) return 128;
   const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128", "256" or "384": testing aid, read per call
@@ -61,10 +66,32 @@ int rows_per_block_16(const xdit_attn_args* a) {
     const int r = std::atoi(force);
     if (r == 128 || r == 256 || r == 384) return r;
   }
+  const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN;
+  const int cus = xdit::resident_cus();
   const int64_t bh = (int64_t)a->B * a->H;
-  if (bh * ((a->Sq + 383) / 384) >= 256) return 384;
-  if (bh * ((a->Sq + 255) / 256) >= 192) return 256;
-  return 128;
+  const int64_t nt = (a->Sk + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile + (a->Sk2 + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile;
+  static const int kRows[3] = {384, 256, 128};
+  static const double kPenalty[3] = {1.0, 1.06, 1.12};
+  int best = 128;
+  double best_cost = 0;
+  for (int i = 0; i < 3; i++) {
+    const int rows = kRows[i];
+    const int per_cu = rows == 128 ? (fp8 ? 3 : 2) : 1;  // workgroups resident per compute unit
+    const int64_t tiles = bh * ((a->Sq + rows - 1) / rows);
+    if (tiles > 0x7fffffff) continue;
+    const int slots = cus * per_cu;
+    xdit::AttnParams q;
+    std::memset(&q, 0, sizeof(q));
+    q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
+    xdit::plan_split(q, rows, slots, 128, 2);
+    const double units = q.split_units ? (double)(q.split_full / slots) * nt + q.split_len + 10
+                                       : (double)((tiles + slots - 1) / slots) * nt;
+    int64_t sharing = (tiles + cus - 1) / cus;  // workgroups on the busiest compute unit at once
+    if (sharing > per_cu) sharing = per_cu;
+    const double cost = units * rows * (double)sharing * kPenalty[i];
+    if (i == 0 || cost < best_cost) { best = rows; best_cost = cost; }
+  }
+  return best;
 }
 
 }  // namespace
