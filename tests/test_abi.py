@@ -32,14 +32,16 @@ def test_library_exports_every_declared_symbol():
 def test_ctypes_structs_match_header(tmp_path):
     c = tmp_path / "sz.c"
     c.write_text('#include "xdit_amd_attn.h"\n#include <stdio.h>\n#include <stddef.h>\n'
-                 'int main(){printf("%zu %zu %zu %zu %zu %zu\\n", sizeof(xdit_attn_args), sizeof(xdit_merge_args),'
+                 'int main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(xdit_attn_args), sizeof(xdit_merge_args),'
                  ' sizeof(xdit_quant_args), offsetof(xdit_attn_args, q_stride), offsetof(xdit_attn_args, stream),'
-                 ' offsetof(xdit_merge_args, acc_lse_stride));}\n')
+                 ' offsetof(xdit_merge_args, acc_lse_stride), sizeof(xdit_prologue_args),'
+                 ' offsetof(xdit_prologue_args, x_stride), offsetof(xdit_quant_args, hadamard_block));}\n')
     exe = tmp_path / "sz"
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(c), "-o", str(exe)])
     got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
     assert got == [ctypes.sizeof(_lib.AttnArgs), ctypes.sizeof(_lib.MergeArgs), ctypes.sizeof(_lib.QuantArgs),
-                   _lib.AttnArgs.q_stride.offset, _lib.AttnArgs.stream.offset, _lib.MergeArgs.acc_lse_stride.offset]
+                   _lib.AttnArgs.q_stride.offset, _lib.AttnArgs.stream.offset, _lib.MergeArgs.acc_lse_stride.offset,
+                   ctypes.sizeof(_lib.PrologueArgs), _lib.PrologueArgs.x_stride.offset, _lib.QuantArgs.hadamard_block.offset]
 
 
 def _attn_args(**kw):
@@ -112,3 +114,83 @@ def test_error_message_is_per_thread_and_cleared_on_entry():
     t = threading.Thread(target=other)
     t.start(); t.join()
     assert seen["msg"] == "" and _lib.last_error() == "args is NULL"
+
+
+def _quant_args(**kw):
+    a = _lib.QuantArgs()
+    a.struct_size = ctypes.sizeof(_lib.QuantArgs)
+    a.in_dtype = _lib.DTYPE_BF16
+    a.B, a.H, a.D, a.S = 1, 2, 128, 64
+    a.x = a.y = a.descale = 0x1000
+    a.x_stride = a.y_stride = _lib.Strides(2 * 64 * 128, 64 * 128, 128)
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize("kw,needle", [
+    (dict(hadamard_block=48), "hadamard_block"),
+    (dict(hadamard_block=256), "hadamard_block"),
+    (dict(hadamard_block=-2), "hadamard_block"),
+    (dict(D=96, hadamard_block=64), "hadamard_block"),
+    (dict(D=4096), "head_dim"),
+    (dict(descale=0), "descale"),
+    (dict(y=0x1004), "8-byte aligned"),
+])
+def test_quant_rejects_bad_arguments(kw, needle):
+    rc = _lib.lib().xdit_fp8_quant(ctypes.byref(_quant_args(**kw)))
+    assert rc == _lib.XDIT_ERR_INVALID_ARG and needle in _lib.last_error()
+
+
+def _prologue_args(**kw):
+    a = _lib.PrologueArgs()
+    a.struct_size = ctypes.sizeof(_lib.PrologueArgs)
+    a.dtype = _lib.DTYPE_BF16
+    a.norm, a.rope = _lib.NORM_HEAD, _lib.ROPE_INTERLEAVED
+    a.B, a.H, a.D, a.S = 1, 2, 128, 64
+    a.eps = 1e-6
+    a.x = a.y = a.weight = a.cos = a.sin = 0x1000
+    a.rope_stride, a.rope_row0, a.rope_rows = 128, 0, 64
+    a.x_stride = a.y_stride = _lib.Strides(2 * 64 * 128, 64 * 128, 128)
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize("kw,code,needle", [
+    (dict(struct_size=8), _lib.XDIT_ERR_INVALID_ARG, "struct_size"),
+    (dict(dtype=_lib.DTYPE_FP8_E4M3FN), _lib.XDIT_ERR_INVALID_ARG, "dtype"),
+    (dict(norm=7), _lib.XDIT_ERR_INVALID_ARG, "norm mode"),
+    (dict(rope=9), _lib.XDIT_ERR_INVALID_ARG, "rope mode"),
+    (dict(D=100), _lib.XDIT_ERR_UNSUPPORTED, "head_dim"),
+    (dict(D=1024), _lib.XDIT_ERR_UNSUPPORTED, "head_dim"),
+    (dict(eps=float("nan")), _lib.XDIT_ERR_INVALID_ARG, "eps"),
+    (dict(cos=0), _lib.XDIT_ERR_INVALID_ARG, "cos / sin are NULL"),
+    (dict(rope_stride=126), _lib.XDIT_ERR_INVALID_ARG, "row stride"),
+    (dict(rope_row0=10, rope_rows=60), _lib.XDIT_ERR_INVALID_ARG, "rope rows"),
+    (dict(weight=0x1002), _lib.XDIT_ERR_INVALID_ARG, "weight"),
+    (dict(norm=_lib.NORM_TOKEN, H=80), _lib.XDIT_ERR_UNSUPPORTED, "token-wide norm supports"),
+    (dict(norm=_lib.NORM_TOKEN, D=72, x_stride=_lib.Strides(2 * 64 * 72, 64 * 72, 72), y_stride=_lib.Strides(2 * 64 * 72, 64 * 72, 72)),
+     _lib.XDIT_ERR_UNSUPPORTED, "token-wide norm needs"),
+    (dict(rope=_lib.ROPE_SPLIT_HALF, D=72, rope_stride=72, x_stride=_lib.Strides(2 * 64 * 72, 64 * 72, 72),
+          y_stride=_lib.Strides(2 * 64 * 72, 64 * 72, 72)), _lib.XDIT_ERR_UNSUPPORTED, "split-half"),
+    (dict(y=0), _lib.XDIT_ERR_INVALID_ARG, "y is NULL"),
+])
+def test_prologue_rejects_bad_arguments(kw, code, needle):
+    L = _lib.lib()
+    assert L.xdit_qk_prologue(None) == _lib.XDIT_ERR_INVALID_ARG
+    rc = L.xdit_qk_prologue(ctypes.byref(_prologue_args(**kw)))
+    assert rc == code and needle in _lib.last_error()
+
+
+def test_workspace_query_needs_no_gpu():
+    """Sizing the balanced-launch workspace is host arithmetic: Flux-1024 at 384 query rows shares
+    the last 32 of its 288 query tiles between 256 workgroups."""
+    a = _attn_args(B=1, H=24, Sq=4608, Sk=4608)
+    for s in ("q_stride", "k_stride", "v_stride", "out_stride"):
+        setattr(a, s, _lib.Strides(24 * 4608 * 128, 4608 * 128, 128))
+    os.environ.pop("XDIT_ATTN_ROWS", None)
+    need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
+    assert need == 32 * (72 // 9 + 1) * 384 * (128 * 2 + 4)
+    a.Sk = 64   # a single KV tile cannot be shared
+    assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) == 0
