@@ -221,6 +221,13 @@ typedef struct {
 
 int xdit_qk_prologue(const xdit_prologue_args* args);
 
+/*
+ * `count` (1..8) prologue jobs in ONE launch: the Q, K and V tensors of the text and image streams
+ * of an attention block (what transformer_flux.py:116-147 handles with some ten separate torch
+ * kernels).  All jobs share dtype and stream; XDIT_NORM_TOKEN jobs cannot be batched.
+ */
+int xdit_qk_prologue_batch(const xdit_prologue_args* jobs, int32_t count);
+
 /* Message of the last error on the calling thread ("" if none). Never NULL. */
 const char* xdit_attn_last_error(void);
 

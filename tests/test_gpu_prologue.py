@@ -149,6 +149,26 @@ def test_flux_joint_qkv_equals_processor_steps_and_feeds_attention(gpu):
     assert (o.double().cpu() - ro).abs().max().item() <= 2e-2 and (l.double().cpu() - rl).abs().max().item() <= 2e-3
 
 
+def test_batch_equals_single_launches(gpu):
+    """One launch of several jobs gives the bits of the separate launches."""
+    g = torch.Generator().manual_seed(11)
+    xs = [torch.randn(1, s, 6, 128, generator=g).bfloat16().to(gpu) for s in (40, 300, 7)]
+    w = (0.8 + 0.4 * torch.rand(128, generator=g)).bfloat16().to(gpu)
+    cos, sin = (t.to(gpu) for t in O.rope_tables(300, 128, seed=3))
+    jobs = [dict(x=xs[0].transpose(1, 2), weight=w, norm="head", rotary_emb=(cos[:40], sin[:40])),
+            dict(x=xs[1].transpose(1, 2), weight=w, norm="head", rotary_emb=(cos, sin), rope="wan"),
+            dict(x=xs[2].transpose(1, 2))]
+    got = ops.qk_prologue_batch(jobs)
+    for j, o in zip(jobs, got):
+        assert torch.equal(o, ops.qk_prologue(**j))
+    with pytest.raises(ValueError):
+        ops.qk_prologue_batch([])
+    with pytest.raises(ValueError):
+        ops.qk_prologue_batch([dict(x=xs[0].transpose(1, 2)), dict(x=xs[1].transpose(1, 2).half())])
+    with pytest.raises(NotImplementedError):
+        ops.qk_prologue_batch([dict(x=xs[0].transpose(1, 2), norm="token")])
+
+
 def test_relayout_only_and_argument_checks(gpu):
     x = torch.randn(2, 50, 6, 64, device=gpu).half()
     y = ops.qk_prologue(x.transpose(1, 2))

@@ -138,7 +138,7 @@ class PrologueArgs(ctypes.Structure):
 NORM_NONE, NORM_HEAD, NORM_TOKEN = 0, 1, 2
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_SPLIT_HALF, ROPE_WAN = 0, 1, 2, 3
 
-EXPORTS = ("xdit_attn_fwd", "xdit_attn_workspace_bytes", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_attn_last_error", "xdit_attn_abi_version")
+EXPORTS = ("xdit_attn_fwd", "xdit_attn_workspace_bytes", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_qk_prologue_batch", "xdit_attn_last_error", "xdit_attn_abi_version")
 
 _lib = None
 _lock = threading.Lock()
@@ -168,6 +168,8 @@ def lib():
         L.xdit_fp8_quant.restype = ctypes.c_int
         L.xdit_qk_prologue.argtypes = [ctypes.POINTER(PrologueArgs)]
         L.xdit_qk_prologue.restype = ctypes.c_int
+        L.xdit_qk_prologue_batch.argtypes = [ctypes.POINTER(PrologueArgs), ctypes.c_int32]
+        L.xdit_qk_prologue_batch.restype = ctypes.c_int
         L.xdit_attn_last_error.argtypes = []
         L.xdit_attn_last_error.restype = ctypes.c_char_p
         L.xdit_attn_abi_version.argtypes = []

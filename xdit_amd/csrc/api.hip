@@ -94,6 +94,59 @@ int rows_per_block_16(const xdit_attn_args* a) {
   return best;
 }
 
+// Validates one prologue job and fills the kernel parameters.
+int fill_prologue(const xdit_prologue_args* a, xdit::PrologueParams& p) {
+  if (a->struct_size != sizeof(xdit_prologue_args))
+    return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_prologue_args));
+  if (a->dtype != XDIT_DTYPE_BF16 && a->dtype != XDIT_DTYPE_FP16 && a->dtype != XDIT_DTYPE_FP32)
+    return fail(XDIT_ERR_INVALID_ARG, "dtype %d must be bf16, fp16 or fp32", a->dtype);
+  if (a->B <= 0 || a->H <= 0 || a->S <= 0) return fail(XDIT_ERR_INVALID_ARG, "B, H, S must be positive");
+  if (a->S > (int64_t(1) << 30) || (int64_t)a->B * a->H * a->S > (int64_t(1) << 40))
+    return fail(XDIT_ERR_INVALID_ARG, "tensor too large for one launch");
+  if (a->D <= 0 || a->D % 8 != 0 || a->D > 512) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d: need a multiple of 8, at most 512", a->D);
+  if (a->norm < XDIT_NORM_NONE || a->norm > XDIT_NORM_TOKEN) return fail(XDIT_ERR_INVALID_ARG, "unknown norm mode %d", a->norm);
+  if (a->rope < XDIT_ROPE_NONE || a->rope > XDIT_ROPE_WAN) return fail(XDIT_ERR_INVALID_ARG, "unknown rope mode %d", a->rope);
+  if (a->norm != XDIT_NORM_NONE && !(a->eps >= 0.f && std::isfinite(a->eps))) return fail(XDIT_ERR_INVALID_ARG, "eps must be finite and >= 0");
+  const int es = elem_size(a->dtype);
+  int rc;
+  if ((rc = check_tensor("x", a->x, a->x_stride, es, a->D))) return rc;
+  if ((rc = check_tensor("y", a->y, a->y_stride, es, a->D))) return rc;
+  if (a->weight != nullptr && !aligned16(a->weight)) return fail(XDIT_ERR_INVALID_ARG, "weight is not 16-byte aligned");
+  const int cpr = a->D / 8;
+  const bool cpr_pow2 = (cpr & (cpr - 1)) == 0;
+  if (a->norm == XDIT_NORM_TOKEN) {
+    if (!cpr_pow2 || cpr > 64) return fail(XDIT_ERR_UNSUPPORTED, "token-wide norm needs head_dim/8 to be a power of two <= 64 (head_dim %d)", a->D);
+    if ((int64_t)a->H * a->D > xdit::prologue_max_token_elems())
+      return fail(XDIT_ERR_UNSUPPORTED, "token-wide norm supports H*D <= %d (got %lld)", xdit::prologue_max_token_elems(), (long long)a->H * a->D);
+  }
+  if (a->rope != XDIT_ROPE_NONE) {
+    if (a->cos == nullptr || a->sin == nullptr) return fail(XDIT_ERR_INVALID_ARG, "cos / sin are NULL");
+    if (!aligned16(a->cos) || !aligned16(a->sin) || a->rope_stride % 4 != 0 || a->rope_stride < 0)
+      return fail(XDIT_ERR_INVALID_ARG, "cos / sin must be 16-byte aligned with a row stride that is a non-negative multiple of 4");
+    if (a->rope_row0 < 0 || a->rope_rows < 0 || a->rope_row0 + a->rope_rows > a->S)
+      return fail(XDIT_ERR_INVALID_ARG, "rope rows [%lld, %lld) do not lie within S=%lld", (long long)a->rope_row0, (long long)(a->rope_row0 + a->rope_rows), (long long)a->S);
+    if (a->rope == XDIT_ROPE_SPLIT_HALF && (!cpr_pow2 || cpr < 2 || cpr > 64))
+      return fail(XDIT_ERR_UNSUPPORTED, "split-half rotation needs head_dim/8 to be a power of two in [2, 64] (head_dim %d)", a->D);
+  }
+  std::memset(&p, 0, sizeof(p));
+  p.x = a->x; p.y = a->y; p.weight = a->norm != XDIT_NORM_NONE ? a->weight : nullptr;
+  p.cos = a->cos; p.sin = a->sin;
+  p.xs_b = a->x_stride.b; p.xs_h = a->x_stride.h; p.xs_s = a->x_stride.s;
+  p.ys_b = a->y_stride.b; p.ys_h = a->y_stride.h; p.ys_s = a->y_stride.s;
+  p.rope_stride = a->rope_stride;
+  p.B = a->B; p.H = a->H; p.S = (int)a->S; p.D = a->D;
+  p.rows = (int64_t)a->B * a->S * a->H;
+  p.norm = a->norm; p.rope_mode = a->rope;
+  p.rope_row0 = (int)a->rope_row0; p.rope_rows = (int)a->rope_rows;
+  int lpr = 1;
+  while (lpr < cpr) lpr <<= 1;
+  p.lpr = lpr;
+  if ((p.rows * lpr + 255) / 256 > 0x7fffffffLL) return fail(XDIT_ERR_INVALID_ARG, "tensor too large for one launch");
+  p.eps = a->eps;
+  p.inv_n = 1.0f / (float)(a->norm == XDIT_NORM_TOKEN ? (int64_t)a->H * a->D : (int64_t)a->D);
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -268,56 +321,31 @@ int xdit_fp8_quant(const xdit_quant_args* a) {
 int xdit_qk_prologue(const xdit_prologue_args* a) {
   g_err[0] = 0;
   if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
-  if (a->struct_size != sizeof(xdit_prologue_args))
-    return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_prologue_args));
-  if (a->dtype != XDIT_DTYPE_BF16 && a->dtype != XDIT_DTYPE_FP16 && a->dtype != XDIT_DTYPE_FP32)
-    return fail(XDIT_ERR_INVALID_ARG, "dtype %d must be bf16, fp16 or fp32", a->dtype);
-  if (a->B <= 0 || a->H <= 0 || a->S <= 0) return fail(XDIT_ERR_INVALID_ARG, "B, H, S must be positive");
-  if (a->S > (int64_t(1) << 30) || (int64_t)a->B * a->H * a->S > (int64_t(1) << 40))
-    return fail(XDIT_ERR_INVALID_ARG, "tensor too large for one launch");
-  if (a->D <= 0 || a->D % 8 != 0 || a->D > 512) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d: need a multiple of 8, at most 512", a->D);
-  if (a->norm < XDIT_NORM_NONE || a->norm > XDIT_NORM_TOKEN) return fail(XDIT_ERR_INVALID_ARG, "unknown norm mode %d", a->norm);
-  if (a->rope < XDIT_ROPE_NONE || a->rope > XDIT_ROPE_WAN) return fail(XDIT_ERR_INVALID_ARG, "unknown rope mode %d", a->rope);
-  if (a->norm != XDIT_NORM_NONE && !(a->eps >= 0.f && std::isfinite(a->eps))) return fail(XDIT_ERR_INVALID_ARG, "eps must be finite and >= 0");
-  const int es = elem_size(a->dtype);
-  int rc;
-  if ((rc = check_tensor("x", a->x, a->x_stride, es, a->D))) return rc;
-  if ((rc = check_tensor("y", a->y, a->y_stride, es, a->D))) return rc;
-  if (a->weight != nullptr && !aligned16(a->weight)) return fail(XDIT_ERR_INVALID_ARG, "weight is not 16-byte aligned");
-  const int cpr = a->D / 8;
-  const bool cpr_pow2 = (cpr & (cpr - 1)) == 0;
-  if (a->norm == XDIT_NORM_TOKEN) {
-    if (!cpr_pow2 || cpr > 64) return fail(XDIT_ERR_UNSUPPORTED, "token-wide norm needs head_dim/8 to be a power of two <= 64 (head_dim %d)", a->D);
-    if ((int64_t)a->H * a->D > xdit::prologue_max_token_elems())
-      return fail(XDIT_ERR_UNSUPPORTED, "token-wide norm supports H*D <= %d (got %lld)", xdit::prologue_max_token_elems(), (long long)a->H * a->D);
-  }
-  if (a->rope != XDIT_ROPE_NONE) {
-    if (a->cos == nullptr || a->sin == nullptr) return fail(XDIT_ERR_INVALID_ARG, "cos / sin are NULL");
-    if (!aligned16(a->cos) || !aligned16(a->sin) || a->rope_stride % 4 != 0 || a->rope_stride < 0)
-      return fail(XDIT_ERR_INVALID_ARG, "cos / sin must be 16-byte aligned with a row stride that is a non-negative multiple of 4");
-    if (a->rope_row0 < 0 || a->rope_rows < 0 || a->rope_row0 + a->rope_rows > a->S)
-      return fail(XDIT_ERR_INVALID_ARG, "rope rows [%lld, %lld) do not lie within S=%lld", (long long)a->rope_row0, (long long)(a->rope_row0 + a->rope_rows), (long long)a->S);
-    if (a->rope == XDIT_ROPE_SPLIT_HALF && (!cpr_pow2 || cpr < 2 || cpr > 64))
-      return fail(XDIT_ERR_UNSUPPORTED, "split-half rotation needs head_dim/8 to be a power of two in [2, 64] (head_dim %d)", a->D);
-  }
   xdit::PrologueParams p;
-  std::memset(&p, 0, sizeof(p));
-  p.x = a->x; p.y = a->y; p.weight = a->norm != XDIT_NORM_NONE ? a->weight : nullptr;
-  p.cos = a->cos; p.sin = a->sin;
-  p.xs_b = a->x_stride.b; p.xs_h = a->x_stride.h; p.xs_s = a->x_stride.s;
-  p.ys_b = a->y_stride.b; p.ys_h = a->y_stride.h; p.ys_s = a->y_stride.s;
-  p.rope_stride = a->rope_stride;
-  p.B = a->B; p.H = a->H; p.S = (int)a->S; p.D = a->D;
-  p.rows = (int64_t)a->B * a->S * a->H;
-  p.norm = a->norm; p.rope_mode = a->rope;
-  p.rope_row0 = (int)a->rope_row0; p.rope_rows = (int)a->rope_rows;
-  int lpr = 1;
-  while (lpr < cpr) lpr <<= 1;
-  p.lpr = lpr;
-  if ((p.rows * lpr + 255) / 256 > 0x7fffffffLL) return fail(XDIT_ERR_INVALID_ARG, "tensor too large for one launch");
-  p.eps = a->eps;
-  p.inv_n = 1.0f / (float)(a->norm == XDIT_NORM_TOKEN ? (int64_t)a->H * a->D : (int64_t)a->D);
+  int rc;
+  if ((rc = fill_prologue(a, p))) return rc;
   hipError_t e = xdit::launch_qk_prologue(p, a->dtype, (hipStream_t)a->stream);
+  if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "prologue launch failed: %s", hipGetErrorString(e));
+  return XDIT_OK;
+}
+
+int xdit_qk_prologue_batch(const xdit_prologue_args* jobs, int32_t count) {
+  g_err[0] = 0;
+  if (jobs == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
+  if (count < 1 || count > xdit::kPrologueBatchMax)
+    return fail(XDIT_ERR_INVALID_ARG, "count %d must be between 1 and %d", count, xdit::kPrologueBatchMax);
+  xdit::PrologueBatch b;
+  std::memset(&b, 0, sizeof(b));
+  b.n = count;
+  for (int i = 0; i < count; i++) {
+    int rc;
+    if ((rc = fill_prologue(&jobs[i], b.job[i]))) return rc;
+    if (jobs[i].dtype != jobs[0].dtype || jobs[i].stream != jobs[0].stream)
+      return fail(XDIT_ERR_INVALID_ARG, "job %d: every job of a batch must have the dtype and the stream of job 0", i);
+    if (jobs[i].norm == XDIT_NORM_TOKEN)
+      return fail(XDIT_ERR_UNSUPPORTED, "job %d: the token-wide norm cannot be batched", i);
+  }
+  hipError_t e = xdit::launch_qk_prologue_batch(b, jobs[0].dtype, (hipStream_t)jobs[0].stream);
   if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "prologue launch failed: %s", hipGetErrorString(e));
   return XDIT_OK;
 }

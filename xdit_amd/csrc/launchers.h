@@ -59,6 +59,13 @@ struct PrologueParams {
   float eps, inv_n;     // inv_n = 1 / number of elements under one norm statistic
 };
 
+// Up to kPrologueBatchMax prologue jobs of one dtype for a single launch.
+constexpr int kPrologueBatchMax = 8;
+struct PrologueBatch {
+  PrologueParams job[kPrologueBatchMax];
+  int n;
+};
+
 // dtype codes below are the C ABI's xdit_dtype values: 0 bf16, 1 fp16, 2 fp32, 3 fp8 e4m3fn.
 hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream);
 size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block);
@@ -67,6 +74,7 @@ size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block);
 hipError_t launch_attn_fwd_f32(const AttnParams& p, int dtype, int D, hipStream_t stream);
 hipError_t launch_fp8_quant(const QuantParams& p, int in_dtype, hipStream_t stream);
 hipError_t launch_qk_prologue(const PrologueParams& p, int dtype, hipStream_t stream);
+hipError_t launch_qk_prologue_batch(const PrologueBatch& b, int dtype, hipStream_t stream);
 int prologue_max_token_elems();
 hipError_t launch_lse_merge(const MergeParams& p, int block_dtype, int final_dtype, hipStream_t stream);
 

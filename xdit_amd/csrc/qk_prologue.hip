@@ -124,7 +124,7 @@ __device__ __forceinline__ float row_sum(float x, int lpr) {
 constexpr int kRowsInFlight = 4;
 
 template <typename T>
-__global__ __launch_bounds__(256) void prologue_rows_kernel(const PrologueParams p) {
+__device__ __forceinline__ void prologue_rows(const PrologueParams& p) {
   const int64_t tok = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6;
   if (tok >= (int64_t)p.B * p.S) return;  // whole wavefronts leave together
   const int lane = threadIdx.x & 63;
@@ -188,6 +188,18 @@ __global__ __launch_bounds__(256) void prologue_rows_kernel(const PrologueParams
       if (chunk_live && h < p.H) store8<T>(y + (int64_t)h * p.ys_h, v[u]);
     }
   }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void prologue_rows_kernel(const PrologueParams p) {
+  prologue_rows<T>(p);
+}
+
+// Several tensors in one launch (the Q, K and V of the text and image streams of one attention
+// block): blockIdx.y selects the job, workgroups beyond a job's tokens leave at once.
+template <typename T>
+__global__ __launch_bounds__(256) void prologue_rows_batch_kernel(const PrologueBatch b) {
+  prologue_rows<T>(b.job[blockIdx.y]);
 }
 
 // Across-heads form (the norm statistic runs over all H*D elements of a token and the gain has
@@ -259,7 +271,25 @@ static hipError_t run(const PrologueParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <typename T>
+static hipError_t run_batch(const PrologueBatch& b, hipStream_t stream) {
+  int64_t tokens = 0;
+  for (int i = 0; i < b.n; i++) {
+    const int64_t t = (int64_t)b.job[i].B * b.job[i].S;
+    if (t > tokens) tokens = t;
+  }
+  hipLaunchKernelGGL((prologue_rows_batch_kernel<T>), dim3((unsigned)((tokens + 3) / 4), (unsigned)b.n), dim3(256), 0, stream, b);
+  return hipGetLastError();
+}
+
 }  // namespace prologue
+
+hipError_t launch_qk_prologue_batch(const PrologueBatch& b, int dtype, hipStream_t stream) {
+  if (dtype == 0) return prologue::run_batch<__bf16>(b, stream);
+  if (dtype == 1) return prologue::run_batch<_Float16>(b, stream);
+  if (dtype == 2) return prologue::run_batch<float>(b, stream);
+  return hipErrorInvalidValue;
+}
 
 int prologue_max_token_elems() { return prologue::kChunks * 256 * 8; }
 

@@ -206,16 +206,8 @@ _NORM_MODES = {None: _lib.NORM_NONE, "none": _lib.NORM_NONE, "head": _lib.NORM_H
 _ROPE_MODES = {"interleaved": _lib.ROPE_INTERLEAVED, "split_half": _lib.ROPE_SPLIT_HALF, "wan": _lib.ROPE_WAN}
 
 
-def qk_prologue(x, weight=None, eps=1e-6, norm=None, rotary_emb=None, rope="interleaved",
-                rope_row0=0, rope_rows=None, out=None):
-    """RMSNorm + rotary embedding + re-layout of a logical BHSD tensor in one pass -> `out`
-    (logical BHSD, any strides; a new BHSD-contiguous tensor when omitted).
-
-    `norm`: None, "head" (over head_dim, `weight` has D entries) or "token" (over all heads of a
-    token, `weight` has H*D entries); `weight` is in x's dtype or None.  `rotary_emb` = (cos, sin),
-    fp32 tensors whose last dimension is D and whose rows (all other dimensions flattened) are the
-    positions; rows [rope_row0, rope_row0 + rope_rows) of S are rotated with table row s - rope_row0.
-    """
+def _prologue_job(x, weight, eps, norm, rotary_emb, rope, rope_row0, rope_rows, out, keep):
+    """Argument struct of one prologue job; tensors that must outlive the launch go to `keep`."""
     device = x.device
     _check4("x", x, device)
     B, H, S, D = x.shape
@@ -235,7 +227,6 @@ def qk_prologue(x, weight=None, eps=1e-6, norm=None, rotary_emb=None, rope="inte
     a.eps = float(eps)
     a.x, a.y = x.data_ptr(), out.data_ptr()
     a.x_stride, a.y_stride = _strides(x), _strides(out)
-    keep = []
     if weight is not None and a.norm != _lib.NORM_NONE:
         n = D if a.norm == _lib.NORM_HEAD else H * D
         if weight.dtype != x.dtype or weight.numel() != n or weight.device != device:
@@ -264,6 +255,38 @@ def qk_prologue(x, weight=None, eps=1e-6, norm=None, rotary_emb=None, rope="inte
         a.rope_stride = cos.stride(0)
         a.rope_row0, a.rope_rows = int(rope_row0), int(rope_rows)
     a.stream = _stream(device)
-    with torch.cuda.device(device):
+    return a, out
+
+
+def qk_prologue(x, weight=None, eps=1e-6, norm=None, rotary_emb=None, rope="interleaved",
+                rope_row0=0, rope_rows=None, out=None):
+    """RMSNorm + rotary embedding + re-layout of a logical BHSD tensor in one pass -> `out`
+    (logical BHSD, any strides; a new BHSD-contiguous tensor when omitted).
+
+    `norm`: None, "head" (over head_dim, `weight` has D entries) or "token" (over all heads of a
+    token, `weight` has H*D entries); `weight` is in x's dtype or None.  `rotary_emb` = (cos, sin),
+    fp32 tensors whose last dimension is D and whose rows (all other dimensions flattened) are the
+    positions; rows [rope_row0, rope_row0 + rope_rows) of S are rotated with table row s - rope_row0.
+    """
+    keep = []
+    a, out = _prologue_job(x, weight, eps, norm, rotary_emb, rope, rope_row0, rope_rows, out, keep)
+    with torch.cuda.device(x.device):
         _lib.check(_lib.lib().xdit_qk_prologue(ctypes.byref(a)))
     return out
+
+
+def qk_prologue_batch(jobs):
+    """Up to 8 prologue jobs of one dtype on one device in ONE launch.  Each job is a dict of the
+    keyword arguments of `qk_prologue` (with `x`).  Returns the list of outputs."""
+    if not 1 <= len(jobs) <= 8:
+        raise ValueError("a batch holds 1 to 8 jobs")
+    keep, outs = [], []
+    arr = (_lib.PrologueArgs * len(jobs))()
+    for i, j in enumerate(jobs):
+        a, out = _prologue_job(j["x"], j.get("weight"), j.get("eps", 1e-6), j.get("norm"), j.get("rotary_emb"),
+                               j.get("rope", "interleaved"), j.get("rope_row0", 0), j.get("rope_rows"), j.get("out"), keep)
+        arr[i] = a
+        outs.append(out)
+    with torch.cuda.device(jobs[0]["x"].device):
+        _lib.check(_lib.lib().xdit_qk_prologue_batch(arr, len(jobs)))
+    return outs

@@ -97,12 +97,12 @@ def flux_joint_qkv(query, key, value, encoder_query, encoder_key, encoder_value,
     concatenation along the sequence, rotary embedding over the joint sequence, transpose to
     BHSD.  Inputs are the projection outputs [B,S_img,H*D] and [B,S_txt,H*D]; norm_* are the gain
     vectors (D entries, the tensors' dtype); image_rotary_emb = (cos, sin) of [S_txt+S_img, D].
-    Returns q, k, v as BHSD-contiguous [B,H,S_txt+S_img,D]: six launches, no intermediate tensor."""
+    Returns q, k, v as BHSD-contiguous [B,H,S_txt+S_img,D]: ONE launch of six jobs, no intermediate tensor."""
     B, S_img, HD = query.shape
     S_txt = encoder_query.shape[1]
     D = HD // heads
     cos, sin = image_rotary_emb
-    outs = []
+    outs, jobs = [], []
     for img, txt, w_img, w_txt, is_v in ((query, encoder_query, norm_q, norm_added_q, False),
                                          (key, encoder_key, norm_k, norm_added_k, False),
                                          (value, encoder_value, None, None, True)):
@@ -110,10 +110,11 @@ def flux_joint_qkv(query, key, value, encoder_query, encoder_key, encoder_value,
         for src, w, row0 in ((txt, w_txt, 0), (img, w_img, S_txt)):
             xb = src.unflatten(-1, (heads, D)).transpose(1, 2)
             n = xb.shape[2]
-            if is_v:
-                ops.qk_prologue(xb, out=out[:, :, row0:row0 + n])
-            else:
-                ops.qk_prologue(xb, weight=w, eps=eps, norm="head", rotary_emb=(cos[row0:row0 + n], sin[row0:row0 + n]),
-                                rope="interleaved", out=out[:, :, row0:row0 + n])
+            job = dict(x=xb, out=out[:, :, row0:row0 + n])
+            if not is_v:
+                job.update(weight=w, eps=eps, norm="head", rotary_emb=(cos[row0:row0 + n], sin[row0:row0 + n]),
+                           rope="interleaved")
+            jobs.append(job)
         outs.append(out)
+    ops.qk_prologue_batch(jobs)
     return tuple(outs)
