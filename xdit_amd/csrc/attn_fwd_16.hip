@@ -338,8 +338,8 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_
   hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, NW>), grid, dim3(64 * NW), lds, stream, q);
   if (q.split_units) {
     const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-    const int64_t threads = (int64_t)(q.total_tiles - q.split_full) * rows * (D / 8);
-    hipLaunchKernelGGL((attn_combine_kernel<T, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, q, rows, nt);
+    const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
+    hipLaunchKernelGGL((attn_combine_kernel<T, D>), cgrid, dim3(256), 0, stream, q, rows, nt);
   }
   return hipGetLastError();
 }

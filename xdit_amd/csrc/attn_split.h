@@ -48,16 +48,16 @@ __device__ __forceinline__ void run_workgroup(const AttnParams& p, Seg seg) {
 
 // Folds the parts of every query tile that was split: out = sum_k exp(lse_k - L) out_k,
 // L = log sum_k exp(lse_k), in fp32; one thread per 8 head_dim elements of a row.
+// grid = (ceil(rows_per_block * D/8 / 256), shared query tiles): blockIdx.y is the tile, so the
+// tile's coordinates and part range are wavefront-uniform.
 template <typename T, int D>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, const int rows_per_block, const int nt) {
   constexpr int TPR = D / 8;
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int rem_tiles = p.total_tiles - p.split_full;
-  const int64_t rrow = gid / TPR;  // row index within the remaining tiles
-  const int col = (int)(gid - rrow * TPR) * 8;
-  if (rrow >= (int64_t)rem_tiles * rows_per_block) return;
-  const int r = (int)(rrow / rows_per_block);
-  const int row = (int)(rrow - (int64_t)r * rows_per_block);
+  const int r = blockIdx.y;  // which of the shared query tiles
+  const int local = blockIdx.x * 256 + threadIdx.x;
+  const int row = local / TPR;
+  const int col = (local - row * TPR) * 8;
+  if (row >= rows_per_block) return;
   const int tile = p.split_full + r;
   const int bh = tile / p.nq_tiles;
   const int qt = tile - bh * p.nq_tiles;
