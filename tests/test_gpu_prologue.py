@@ -187,3 +187,21 @@ def test_relayout_only_and_argument_checks(gpu):
         ops.qk_prologue(torch.zeros(1, 2, 4, 72, device=gpu), rotary_emb=(torch.ones(4, 72, device=gpu),) * 2, rope="split_half")
     with pytest.raises(RuntimeError, match="no CPU path"):
         ops.qk_prologue(torch.zeros(1, 2, 4, 64))
+
+
+def test_norm_rope_custom_op(gpu):
+    from xdit_amd import custom_ops  # noqa: F401
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(1, 60, 4, 128, generator=g).bfloat16().to(gpu).transpose(1, 2)
+    w = (0.8 + 0.4 * torch.rand(128, generator=g)).bfloat16().to(gpu)
+    cos, sin = (t.to(gpu) for t in O.rope_tables(60, 128, seed=2))
+    args = (x, w, cos, sin, 1e-6, "head", "interleaved", 0, 60)
+    torch.library.opcheck(torch.ops.xdit_amd.norm_rope.default, args,
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+    eager = ops.qk_prologue(x, weight=w, norm="head", rotary_emb=(cos, sin))
+    assert torch.equal(torch.ops.xdit_amd.norm_rope(*args), eager)
+    fn = torch.compile(lambda a: torch.ops.xdit_amd.norm_rope(a * 1, w, cos, sin, 1e-6, "head", "interleaved", 0, 60) + 0,
+                       backend="aot_eager", fullgraph=True)
+    assert torch.equal(fn(x), eager)
+    plain = torch.ops.xdit_amd.norm_rope(x, w, cos, sin, 0.0, "none", "none", 0, 0)
+    assert torch.equal(plain, x.contiguous())

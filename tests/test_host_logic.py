@@ -142,6 +142,10 @@ def test_custom_ops_fake_implementations_describe_the_outputs():
     assert out.dtype == torch.bfloat16
     y, ds = torch.ops.xdit_amd.fp8_quant(q, False, 128)
     assert y.dtype == torch.float8_e4m3fn and y.shape == q.shape and y.is_contiguous() and ds.shape == (B, H)
+    w = torch.empty(D, dtype=torch.bfloat16, device="meta")
+    cs = torch.empty(Sq, D, device="meta")
+    y = torch.ops.xdit_amd.norm_rope(q, w, cs, cs, 1e-6, "head", "interleaved", 0, Sq)
+    assert y.shape == q.shape and y.dtype == q.dtype and y.is_contiguous()
     # there is no CPU implementation behind the ops either
     with pytest.raises((NotImplementedError, RuntimeError)):
         torch.ops.xdit_amd.attn_fwd(torch.zeros(1, 1, 4, 128), torch.zeros(1, 1, 4, 128), torch.zeros(1, 1, 4, 128), 0.1)

@@ -12,6 +12,8 @@ The reference wraps a vendor kernel the same way (xfuser/core/distributed/attent
     xdit_amd::lse_merge       (acc_out, acc_lse, block_out, block_lse, first)   in place
     xdit_amd::lse_merge_final (acc_out, acc_lse, block_out, block_lse, final_out)  in place
     xdit_amd::fp8_quant       (x, per_tensor, hadamard_block)               -> (y, descale)
+    xdit_amd::norm_rope       (x, weight, cos, sin, eps, norm, rope,
+                               rope_row0, rope_rows)                        -> y (BHSD-contiguous)
 
 All tensors are logical BHSD (any B/H/S strides); outputs are BHSD-contiguous, lse is (B,H,Sq)
 fp32.  The ops are registered for GPU tensors only: there is no CPU implementation.
@@ -96,3 +98,19 @@ def _fp8_quant_fake(x, per_tensor, hadamard_block):
     B, H, S, D = x.shape
     return (x.new_empty((B, H, S, D), dtype=torch.float8_e4m3fn),
             x.new_empty((B, H), dtype=torch.float32))
+
+
+@custom_op("xdit_amd::norm_rope", mutates_args=(), device_types="cuda")
+def norm_rope(x: Tensor, weight: Tensor, cos: Tensor, sin: Tensor, eps: float, norm: str, rope: str,
+              rope_row0: int, rope_rows: int) -> Tensor:
+    """Fused RMSNorm + rotary embedding + re-layout of a logical BHSD tensor (`ops.qk_prologue`).
+    `norm` is "none", "head" or "token" (`weight` is ignored for "none": pass any tensor);
+    `rope` is "none", "interleaved", "split_half" or "wan" (`cos`/`sin` ignored for "none")."""
+    return ops.qk_prologue(x, weight=None if norm == "none" else weight, eps=eps, norm=None if norm == "none" else norm,
+                           rotary_emb=None if rope == "none" else (cos, sin), rope="interleaved" if rope == "none" else rope,
+                           rope_row0=rope_row0, rope_rows=rope_rows if rope != "none" else None)
+
+
+@register_fake("xdit_amd::norm_rope")
+def _norm_rope_fake(x, weight, cos, sin, eps, norm, rope, rope_row0, rope_rows):
+    return x.new_empty(tuple(x.shape))
