@@ -241,7 +241,9 @@ __device__ __forceinline__ void attn_segment_fp8(const AttnParams& p, unsigned c
         float p2 = fast_exp2(__builtin_fmaf(sacc[kb][i + 2], c, -mc));
         float p3 = fast_exp2(__builtin_fmaf(sacc[kb][i + 3], c, -mc));
         l_part += (p0 + p1) + (p2 + p3);
-        int w = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
+        int w;  // both halves are written below: no need to clear the register first
+        asm volatile("" : "=v"(w));
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, w, false);
         w = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, w, true);
         pf[4 * kb + (i >> 2)] = w;
       }
