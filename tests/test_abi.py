@@ -194,3 +194,16 @@ def test_workspace_query_needs_no_gpu():
     assert need == 32 * (72 // 9 + 1) * 384 * (128 * 2 + 4)
     a.Sk = 64   # a single KV tile cannot be shared
     assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) == 0
+
+
+def test_workspace_of_claimed_ranges(monkeypatch):
+    """A long share (128 remaining query tiles of 256 KV iterations over 256 workgroups = 128
+    iterations each) is cut into ranges of 64 iterations that workgroups claim one after the
+    other: 4 (+1) slots per remaining tile, plus 256 bytes for the range counter."""
+    monkeypatch.setenv("XDIT_ATTN_ROWS", "384")
+    a = _attn_args(B=1, H=12, Sq=32 * 384, Sk=256 * 64)
+    a.q_stride = a.out_stride = _lib.Strides(12 * 32 * 384 * 128, 32 * 384 * 128, 128)
+    a.k_stride = a.v_stride = _lib.Strides(12 * 256 * 64 * 128, 256 * 64 * 128, 128)
+    need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
+    parts = 128 * (256 // 64 + 1) * 384 * (128 * 2 + 4)
+    assert parts % 256 == 0 and need == parts + 256

@@ -133,6 +133,40 @@ def force_rows(monkeypatch):
     return set_rows
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["bf16", "fp8"])
+def test_claimed_ranges_vs_plain_launch_and_fp32(gpu, force_rows, kind):
+    """384 query tiles of 384 rows over 256 KV iterations: the 128 tiles of the second round are
+    cut into 512 ranges of 64 iterations which the 256 workgroups of the bf16 kernel claim from a
+    counter (the fp8 kernel gives every workgroup one range of 128).  The result must match the
+    plain launch, a fp32 computation of two heads, and itself on a second call (which workgroup
+    takes which range changes nothing)."""
+    force_rows(384)
+    B, H, Sq, Sk = 1, 12, 32 * 384, 256 * 64
+    g = torch.Generator(device=gpu).manual_seed(77)
+    q, k, v = (torch.randn(B, H, n, 128, generator=g, device=gpu) for n in (Sq, Sk, Sk))
+    if kind == "fp8":
+        (q8, qd), (k8, kd), (v8, vd) = (ops.fp8_quant(t.to(torch.bfloat16)) for t in (q, k, v))
+        args, kw = (q8, k8, v8), dict(q_descale=qd, k_descale=kd, v_descale=vd)
+        deq = lambda t, d: t.float() * d[:, :, None, None]
+        qf, kf, vf = deq(q8, qd), deq(k8, kd), deq(v8, vd)
+        tol_o, tol_l = 6e-2, 1e-3
+    else:
+        args, kw = tuple(t.to(torch.bfloat16) for t in (q, k, v)), {}
+        qf, kf, vf = (t.float() for t in args)
+        tol_o, tol_l = TOL[torch.bfloat16]
+    o, l = ops.attn_fwd(*args, **kw)
+    o1, l1 = ops.attn_fwd(*args, balance=False, **kw)
+    assert (o.float() - o1.float()).abs().max().item() <= 1e-2 and (l - l1).abs().max().item() <= 1e-5
+    for h in (0, H - 1):
+        s = (qf[:, h] @ kf[:, h].transpose(-1, -2)) * 128 ** -0.5
+        ro, rl = torch.softmax(s, -1) @ vf[:, h], torch.logsumexp(s, -1)
+        assert (o[:, h].float() - ro).abs().max().item() <= tol_o
+        assert (l[:, h] - rl).abs().max().item() <= tol_l
+    o2, l2 = ops.attn_fwd(*args, **kw)
+    assert torch.equal(o, o2) and torch.equal(l, l2)
+
+
 @pytest.mark.parametrize("rows", [128, 256, 384])
 @pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8"])
 @pytest.mark.parametrize("B,H,Sq,Sk,Sk2", [

@@ -83,8 +83,8 @@ int rows_per_block_16(const xdit_attn_args* a) {
     xdit::AttnParams q;
     std::memset(&q, 0, sizeof(q));
     q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
-    xdit::plan_split(q, rows, slots, 128, 2);
-    const double units = q.split_units ? (double)(q.split_full / slots) * nt + q.split_len + 10
+    xdit::plan_split(q, rows, slots, 128, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup);
+    const double units = q.split_units ? (double)(q.split_full / slots) * nt + q.split_share + 10
                                        : (double)((tiles + slots - 1) / slots) * nt;
     int64_t sharing = (tiles + cus - 1) / cus;  // workgroups on the busiest compute unit at once
     if (sharing > per_cu) sharing = per_cu;

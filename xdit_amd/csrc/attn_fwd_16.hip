@@ -327,8 +327,9 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2), rows, D, 2);
-  dim3 grid(q.split_units ? q.split_full + q.split_units : q.tiles_per_xcd * 8);
+  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup), rows, D, 2);
+  if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
+  dim3 grid(split_grid(q));
   constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
   if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
     hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -351,7 +352,7 @@ static size_t workspace_one(const AttnParams& p) {
   constexpr int rows = 32 * NW;
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
-  return plan_split(q, rows, resident_workgroups(NW), D, 2);
+  return plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup);
 }
 
 size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block) {

@@ -328,8 +328,9 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2), rows, D, 2);
-  dim3 grid(q.split_units ? q.split_full + q.split_units : q.tiles_per_xcd * 8);
+  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2, 1), rows, D, 2);
+  if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
+  dim3 grid(split_grid(q));
   hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW>), grid, dim3(64 * NW), 0, stream, q);
   if (q.split_units) {
     const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
@@ -345,7 +346,7 @@ static size_t workspace_one(const AttnParams& p) {
   constexpr int rows = kRowsPerWave * NW;
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
-  return plan_split(q, rows, resident_workgroups(NW), D, 2);
+  return plan_split(q, rows, resident_workgroups(NW), D, 2, 1);
 }
 
 }  // namespace fp8path

@@ -12,8 +12,15 @@ namespace xdit {
 // Plain launch (split_units == 0): workgroup = one query tile over all KV tiles.  Balanced launch:
 // the first split_full workgroups each take a whole query tile; the KV iterations of the
 // remaining query tiles, laid end to end, are cut into split_units ranges of split_len
-// iterations, one per workgroup.  A range may cover the end of one query tile and the start of
-// the next.  TO is the output element type, ROWS the query rows per workgroup.
+// iterations.  A range may cover the end of one query tile and the start of the next.  The
+// ranges are processed by split_claimers workgroups: the workgroups split_fuse0 .. split_full-1
+// (the last to be dispatched) after their own query tile, so that no compute unit waits for a
+// new workgroup to be dispatched in between, or, with fewer whole tiles than that
+// (split_fuse0 > split_full), workgroups of their own, split_full .. split_full+claimers-1.
+// Claimer c starts with range c; when there are more ranges than claimers (split_counter !=
+// nullptr) every further range is taken from a counter in device memory, so that compute units
+// that run faster (the clocks of the eight XCDs differ by several per cent) take more of them.
+// TO is the output element type, ROWS the query rows per workgroup.
 template <typename TO, int ROWS, int D, typename Seg>
 __device__ __forceinline__ void run_workgroup(const AttnParams& p, Seg seg) {
   const int nt = (p.Sk + kKeysPerTile - 1) / kKeysPerTile + (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
@@ -23,27 +30,43 @@ __device__ __forceinline__ void run_workgroup(const AttnParams& p, Seg seg) {
     seg(tile, 0, nt, (TO*)nullptr, (float*)nullptr);
     return;
   }
+  __shared__ int next_unit;
   const int w = blockIdx.x;
+  int u = w - p.split_full;
+  bool first = true;
   if (w < p.split_full) {
     seg(xcd_tile_index(w, p.split_full >> 3), 0, nt, (TO*)nullptr, (float*)nullptr);
-    return;
-  }
-  const int u = w - p.split_full;
-  const int rem_iters = (p.total_tiles - p.split_full) * nt;
-  int lin = u * p.split_len;
-  const int lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
-  bool first = true;
-  while (lin < lin_end) {
-    const int r = lin / nt;               // which of the remaining query tiles
-    const int it0 = lin - r * nt;
-    const int it1 = (lin_end - r * nt) < nt ? (lin_end - r * nt) : nt;
-    const int part = u - (r * nt) / p.split_len;  // ranges are consecutive: index within the tile
-    const int64_t slot = (int64_t)r * p.split_pmax + part;
-    if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
-    seg(p.split_full + r, it0, it1, (TO*)p.ws_out + slot * ROWS * D, p.ws_lse + slot * ROWS);
+    u = w - p.split_fuse0;
+    if (u < 0) return;
     first = false;
-    lin += it1 - it0;
   }
+  const int rem_iters = (p.total_tiles - p.split_full) * nt;
+  while (u < p.split_units) {
+    int lin = u * p.split_len;
+    const int lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
+    while (lin < lin_end) {
+      const int r = lin / nt;               // which of the remaining query tiles
+      const int it0 = lin - r * nt;
+      const int it1 = (lin_end - r * nt) < nt ? (lin_end - r * nt) : nt;
+      const int part = u - (r * nt) / p.split_len;  // ranges are consecutive: index within the tile
+      const int64_t slot = (int64_t)r * p.split_pmax + part;
+      if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
+      seg(p.split_full + r, it0, it1, (TO*)p.ws_out + slot * ROWS * D, p.ws_lse + slot * ROWS);
+      first = false;
+      lin += it1 - it0;
+    }
+    if (p.split_counter == nullptr) return;
+    __syncthreads();  // everyone has read next_unit of the previous round
+    if (threadIdx.x == 0) next_unit = p.split_claimers + (int)atomicAdd(p.split_counter, 1u);
+    __syncthreads();
+    u = next_unit;
+  }
+}
+
+// Clears the range counter of a balanced launch (a kernel, not a memset, so that the sequence
+// can be captured into a graph).
+static __global__ void attn_counter_reset_kernel(unsigned* counter) {
+  if (threadIdx.x == 0) *counter = 0u;
 }
 
 // Folds the parts of every query tile that was split: out = sum_k exp(lse_k - L) out_k,
@@ -110,40 +133,75 @@ static inline int resident_cus() {
   return cus;
 }
 
+// Ranges shorter than this many KV iterations are not worth a claim of their own (prologue,
+// epilogue and partial result of a segment cost about four iterations).
+constexpr int kMinClaimLen = 64;
+// Ranges per claimer aimed at when ranges are claimed one after the other.  Worth it for the
+// 16-bit kernels, which run power-limited with XCD clocks several per cent apart (HunyuanVideo
+// shard: 18.22 -> 17.85 ms at 6, 17.95 at 4 and at 12); the fp8 kernel runs at equal clocks and
+// only pays for the extra partial results.
+constexpr int kClaimsPerWorkgroup = 6;
+
 // Decide how to balance the launch; fills the split_* fields of q.  Returns the workspace bytes
 // the balanced launch needs (0 = plain launch).
-// `rows` query rows per workgroup, `slots` workgroups resident at once, `out_bytes` per output element.
-static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int out_bytes) {
-  q.split_units = q.split_full = q.split_len = q.split_pmax = 0;
+// `rows` query rows per workgroup, `slots` workgroups resident at once, `out_bytes` per output
+// element, `claims` ranges per workgroup to aim at (1: every workgroup gets one range).
+static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int out_bytes, int claims) {
+  q.split_units = q.split_full = q.split_len = q.split_pmax = q.split_share = q.split_claimers = 0;
+  q.split_fuse0 = 0x7fffffff;
+  q.split_counter = nullptr;
   const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
   const int T = q.total_tiles;
   const int full = (T / slots) * slots;
   const int rem = T - full;
   if (rem == 0 || nt < 8) return 0;
-  int len = (int)(((int64_t)rem * nt + slots - 1) / slots);
-  if (len < 4) len = 4;
+  int share = (int)(((int64_t)rem * nt + slots - 1) / slots);  // iterations per workgroup
+  if (share < 4) share = 4;
   // Iterations of the critical path saved by filling the last round.  Idle CUs leave the busy
   // ones more power (higher clock), so a partly filled round costs less than its length suggests;
   // balance only when the saving clearly exceeds the cost of the extra prologues, the partial
   // results and the combine pass (measured: about 10 iterations' worth).
-  if (nt - len < 48) return 0;
+  if (nt - share < 48) return 0;
+  // Long shares are cut into several ranges that are claimed one after the other.
+  int len = share;
+  if (claims > 1 && share >= 2 * kMinClaimLen) {
+    len = (share + claims - 1) / claims;
+    if (len < kMinClaimLen) len = kMinClaimLen;
+  }
   const int units = (int)(((int64_t)rem * nt + len - 1) / len);
+  const int claimers = units < slots ? units : slots;
   q.split_full = full;
   q.split_units = units;
   q.split_len = len;
+  q.split_share = share;
   q.split_pmax = (nt + len - 1) / len + 1;
-  return (size_t)rem * q.split_pmax * rows * ((size_t)D * out_bytes + 4);
+  q.split_claimers = claimers;
+  q.split_fuse0 = full >= claimers ? full - claimers : 0x7fffffff;
+  const size_t parts = (size_t)rem * q.split_pmax * rows * ((size_t)D * out_bytes + 4);
+  return units > claimers ? ((parts + 255) & ~(size_t)255) + 256 : parts;  // + the range counter
 }
 
-// Point ws_lse behind the partial outputs, or fall back to a plain launch when the caller gave no
-// (or too small a) workspace.
+// Point ws_lse (and the range counter) behind the partial outputs, or fall back to a plain launch
+// when the caller gave no (or too small a) workspace.
 static inline void bind_workspace(AttnParams& q, const AttnParams& p, size_t need, int rows, int D, int out_bytes) {
   if (need == 0 || p.ws_out == nullptr || p.ws_bytes < need) {
-    q.split_units = q.split_full = q.split_len = q.split_pmax = 0;
+    q.split_units = q.split_full = q.split_len = q.split_pmax = q.split_share = q.split_claimers = 0;
+    q.split_fuse0 = 0x7fffffff;
+    q.split_counter = nullptr;
   } else {
-    const int rem = q.total_tiles - q.split_full;
-    q.ws_lse = (float*)((unsigned char*)p.ws_out + (size_t)rem * q.split_pmax * rows * D * out_bytes);
+    const size_t rem = (size_t)(q.total_tiles - q.split_full);
+    q.ws_lse = (float*)((unsigned char*)p.ws_out + rem * q.split_pmax * rows * D * out_bytes);
+    if (q.split_units > q.split_claimers) {
+      const size_t parts = rem * q.split_pmax * rows * ((size_t)D * out_bytes + 4);
+      q.split_counter = (unsigned*)((unsigned char*)p.ws_out + ((parts + 255) & ~(size_t)255));
+    }
   }
+}
+
+// Workgroups of a launch planned by plan_split (after bind_workspace).
+static inline unsigned split_grid(const AttnParams& q) {
+  if (q.split_units == 0) return (unsigned)(q.tiles_per_xcd * 8);
+  return (unsigned)(q.split_fuse0 <= q.split_full ? q.split_full : q.split_full + q.split_claimers);
 }
 
 }  // namespace xdit

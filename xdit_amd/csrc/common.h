@@ -55,6 +55,10 @@ struct AttnParams {
   int split_units;    // workgroups sharing the KV iterations of the remaining query tiles
   int split_len;      // KV iterations per such workgroup
   int split_pmax;     // workspace slots per remaining query tile
+  int split_fuse0;    // first workgroup that takes a range after its own query tile (> split_full: none)
+  int split_share;    // KV iterations of the remaining query tiles per resident workgroup
+  int split_claimers; // workgroups that process ranges
+  unsigned* split_counter;  // ranges handed out beyond the first of every claimer (nullptr: one range each)
   void* ws_out;       // workspace: partial outputs [tile][slot][row][D] in the output dtype ...
   float* ws_lse;      // ... followed by partial log-sum-exps [tile][slot][row]
   size_t ws_bytes;
