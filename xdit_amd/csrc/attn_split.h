@@ -24,42 +24,58 @@ namespace xdit {
 template <typename TO, int ROWS, int D, typename Seg>
 __device__ __forceinline__ void run_workgroup(const AttnParams& p, Seg seg) {
   const int nt = (p.Sk + kKeysPerTile - 1) / kKeysPerTile + (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-  if (p.split_units == 0) {
-    const int tile = xcd_tile_index(blockIdx.x, p.tiles_per_xcd);
-    if (tile >= p.total_tiles) return;
-    seg(tile, 0, nt, (TO*)nullptr, (float*)nullptr);
-    return;
-  }
   __shared__ int next_unit;
   const int w = blockIdx.x;
-  int u = w - p.split_full;
-  bool first = true;
-  if (w < p.split_full) {
-    seg(xcd_tile_index(w, p.split_full >> 3), 0, nt, (TO*)nullptr, (float*)nullptr);
-    u = w - p.split_fuse0;
-    if (u < 0) return;
-    first = false;
+  // What this workgroup does: a whole query tile first (whole_tile >= 0), then ranges (claimer).
+  int whole_tile = -1;
+  int u_next = -1;  // the range to start with, < 0: none
+  if (p.split_units == 0) {
+    whole_tile = xcd_tile_index(w, p.tiles_per_xcd);
+    if (whole_tile >= p.total_tiles) return;
+  } else if (w < p.split_full) {
+    whole_tile = xcd_tile_index(w, p.split_full >> 3);
+    u_next = w - p.split_fuse0;
+  } else {
+    u_next = w - p.split_full;
   }
   const int rem_iters = (p.total_tiles - p.split_full) * nt;
-  while (u < p.split_units) {
-    int lin = u * p.split_len;
-    const int lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
-    while (lin < lin_end) {
+  int u = 0, lin = 0, lin_end = 0;
+  bool first = true;
+  for (;;) {  // one segment per turn; a single call site keeps one copy of the kernel body
+    int tile, it0, it1;
+    TO* part_out = nullptr;
+    float* part_lse = nullptr;
+    if (whole_tile >= 0) {
+      tile = whole_tile; it0 = 0; it1 = nt;
+      whole_tile = -1;
+    } else {
+      if (lin >= lin_end) {  // the next range
+        if (u_next < 0 || u_next >= p.split_units) return;
+        u = u_next;
+        u_next = -1;
+        lin = u * p.split_len;
+        lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
+      }
       const int r = lin / nt;               // which of the remaining query tiles
-      const int it0 = lin - r * nt;
-      const int it1 = (lin_end - r * nt) < nt ? (lin_end - r * nt) : nt;
+      it0 = lin - r * nt;
+      it1 = (lin_end - r * nt) < nt ? (lin_end - r * nt) : nt;
       const int part = u - (r * nt) / p.split_len;  // ranges are consecutive: index within the tile
       const int64_t slot = (int64_t)r * p.split_pmax + part;
-      if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
-      seg(p.split_full + r, it0, it1, (TO*)p.ws_out + slot * ROWS * D, p.ws_lse + slot * ROWS);
-      first = false;
+      tile = p.split_full + r;
+      part_out = (TO*)p.ws_out + slot * ROWS * D;
+      part_lse = p.ws_lse + slot * ROWS;
       lin += it1 - it0;
     }
-    if (p.split_counter == nullptr) return;
-    __syncthreads();  // everyone has read next_unit of the previous round
-    if (threadIdx.x == 0) next_unit = p.split_claimers + (int)atomicAdd(p.split_counter, 1u);
-    __syncthreads();
-    u = next_unit;
+    if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
+    seg(tile, it0, it1, part_out, part_lse);
+    first = false;
+    if (whole_tile < 0 && lin >= lin_end && u_next < 0 && p.split_counter != nullptr && p.split_units != 0 &&
+        (w >= p.split_fuse0 || w >= p.split_full)) {
+      __syncthreads();  // everyone has read next_unit of the previous claim
+      if (threadIdx.x == 0) next_unit = p.split_claimers + (int)atomicAdd(p.split_counter, 1u);
+      __syncthreads();
+      u_next = next_unit;
+    }
   }
 }
 
@@ -92,26 +108,37 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, c
   const int last_unit = ((r + 1) * nt - 1) / p.split_len;
   const int nparts = last_unit - first_unit + 1;
   const float* lsep = p.ws_lse + ((int64_t)r * p.split_pmax) * rows_per_block + row;
-  float L = -INFINITY;
-  for (int k = 0; k < nparts; k++) L = fmaxf(L, lsep[(int64_t)k * rows_per_block]);
-  float denom = 0.f;
-  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   typedef __attribute__((ext_vector_type(8))) T vec8;
   const T* part0 = (const T*)p.ws_out + (((int64_t)r * p.split_pmax) * rows_per_block + row) * D + col;
-  for (int k0 = 0; k0 < nparts; k0 += 4) {  // four parts in flight per thread
-    vec8 x[4];
-    float w[4];
+  // One pass, eight parts in flight per thread (outputs and log-sum-exps are loaded together,
+  // so a tile of up to eight parts costs one round trip to memory); the running maximum L is
+  // carried from one group of eight to the next as in the online softmax.
+  float L = -INFINITY;
+  float denom = 0.f;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < nparts; k0 += 8) {
+    vec8 x[8];
+    float ls[8];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < 8; j++) {
       const int k = k0 + j < nparts ? k0 + j : nparts - 1;
       x[j] = *(const vec8*)(part0 + (int64_t)k * rows_per_block * D);
-      w[j] = k0 + j < nparts ? __expf(lsep[(int64_t)k * rows_per_block] - L) : 0.f;
+      ls[j] = lsep[(int64_t)k * rows_per_block];
     }
+    float Ln = L;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      denom += w[j];
+    for (int j = 0; j < 8; j++) Ln = fmaxf(Ln, ls[j]);
+    const float keep = __expf(L - Ln);  // 0 on the first group (L = -inf)
+    L = Ln;
+    denom *= keep;
 #pragma unroll
-      for (int i = 0; i < 8; i++) acc[i] += w[j] * (float)x[j][i];
+    for (int i = 0; i < 8; i++) acc[i] *= keep;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float w = k0 + j < nparts ? __expf(ls[j] - L) : 0.f;
+      denom += w;
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[i] += w * (float)x[j][i];
     }
   }
   const float inv = 1.0f / denom;
