@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define XDIT_ATTN_ABI_VERSION 3
+#define XDIT_ATTN_ABI_VERSION 4
 
 typedef enum {
   XDIT_OK = 0,
@@ -139,6 +139,36 @@ typedef struct {
 } xdit_merge_args;
 
 int xdit_lse_merge(const xdit_merge_args* args);
+
+/*
+ * One ring step in one launch: the forward of xdit_attn_fwd on this step's keys/values, folded
+ * into the fp32 accumulator (acc_out, acc_lse) in the kernel's epilogue with the arithmetic of
+ * xdit_lse_merge.  The block's rows are rounded to `dtype` before the fold, as if they had gone
+ * through a block_out tensor, so the result equals xdit_attn_fwd + xdit_lse_merge bit for bit
+ * while the block is never written to memory and the accumulator is touched once.
+ *   first != 0            initialise the accumulator from this block (acc_out is not read)
+ *   args->out  (or NULL)  receives the merged rows in out_dtype: the final step's cast
+ *   args->lse  (or NULL)  receives the merged log-sum-exp, (B,H,Sq) with args' lse strides
+ *   discard_acc_out != 0  acc_out is read but not written back (last step: `out` and acc_lse
+ *                         carry the result); needs args->out
+ * acc_out is logical (B,H,Sq,D) fp32, acc_lse logical (B,H,Sq) fp32 with its own strides (the
+ * (B,S,H,1) accumulator of the legacy ring maps without a copy).  bf16 / fp16 inputs with
+ * head_dim 64 or 128; XDIT_ERR_UNSUPPORTED otherwise (use the two calls).  args->workspace is
+ * not used.
+ * Replaces, per ring step: the kernel call at ring_flash_attn.py:123-134, update_out_and_lse at
+ * :138 and, on the last step, the cast at :145.
+ */
+typedef struct {
+  uint32_t struct_size;        /* = sizeof(xdit_ring_acc) */
+  int32_t first;
+  int32_t discard_acc_out;
+  int32_t reserved0;
+  float* acc_out;
+  float* acc_lse;
+  xdit_strides acc_out_stride, acc_lse_stride;
+} xdit_ring_acc;
+
+int xdit_attn_fwd_accumulate(const xdit_attn_args* args, const xdit_ring_acc* acc);
 
 /*
  * Abs-max fp8 quantiser, the step in front of the fp8 forward:

@@ -207,3 +207,29 @@ def test_workspace_of_claimed_ranges(monkeypatch):
     need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
     parts = 128 * (256 // 64 + 1) * 384 * (128 * 2 + 4)
     assert parts % 256 == 0 and need == parts + 256
+
+
+def test_fused_ring_step_rejects_bad_arguments():
+    """xdit_attn_fwd_accumulate validates before it launches: no GPU needed for the error paths."""
+    L = _lib.lib()
+    a = _attn_args()
+    assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), None) == _lib.XDIT_ERR_INVALID_ARG and "acc is NULL" in _lib.last_error()
+    r = _lib.RingAcc()
+    r.struct_size = 8
+    assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "acc struct_size" in _lib.last_error()
+    r.struct_size = ctypes.sizeof(_lib.RingAcc)
+    assert ctypes.sizeof(_lib.RingAcc) == 16 + 16 + 2 * 24
+    r.acc_out, r.acc_lse = 0x2000, 0x3000
+    r.acc_out_stride = _lib.Strides(a.H * a.Sq * a.D, a.Sq * a.D, a.D)
+    r.acc_lse_stride = _lib.Strides(a.H * a.Sq, a.Sq, 1)
+    f8 = _attn_args(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16)
+    assert L.xdit_attn_fwd_accumulate(ctypes.byref(f8), ctypes.byref(r)) == _lib.XDIT_ERR_UNSUPPORTED and "fused ring step" in _lib.last_error()
+    r.acc_out = 0x2004
+    assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "acc_out" in _lib.last_error()
+    r.acc_out = 0x2000
+    r.acc_lse = 0
+    assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "acc_lse is NULL" in _lib.last_error()
+    r.acc_lse = 0x3000
+    r.discard_acc_out = 1
+    a.out = 0
+    assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "discard_acc_out" in _lib.last_error()

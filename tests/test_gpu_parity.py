@@ -391,6 +391,107 @@ def test_update_out_and_lse_matches_oracle_layout(gpu):
     assert _err(out, rout) <= 5e-6 and _err(lse, rlse) <= 5e-6
 
 
+# ---------------------------------------------------------------------------- fused ring step
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64)])
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+def test_fused_ring_step_equals_forward_plus_merge(gpu, force_rows, dtype, D, layout):
+    """xdit_attn_fwd_accumulate = xdit_attn_fwd + xdit_lse_merge, bit for bit, over three steps
+    (initialise, fold, fold with the final cast), in both memory layouts, with the ragged sizes
+    and every workgroup shape; against the oracle's fold as well."""
+    B, H, Sq = 2, 3, 333
+    g = torch.Generator().manual_seed(D + Sq)
+    q = torch.randn(B, H, Sq, D, generator=g).to(dtype)
+    chunks = [(torch.randn(B, H, n, D, generator=g).to(dtype), torch.randn(B, H, n, D, generator=g).to(dtype)) for n in (257, 64, 130)]
+    for rows in ((128, 256, 384) if D == 128 else (128,)):
+        force_rows(rows)
+        qd = _layout(q, layout, gpu)
+        acc_o = _layout(torch.full((B, H, Sq, D), float("nan")), layout, gpu)
+        acc_l = torch.full((B, Sq, H, 1), float("nan"), device=gpu).squeeze(-1).transpose(1, 2)  # legacy (B,S,H,1) layout
+        ref_o = torch.empty(B, H, Sq, D, device=gpu)
+        ref_l = torch.empty(B, H, Sq, device=gpu)
+        fin = torch.empty(B, H, Sq, D, dtype=dtype, device=gpu)
+        ref_fin = torch.empty_like(fin)
+        oo = ol = None
+        for i, (k, v) in enumerate(chunks):
+            kd, vd = _layout(k, layout, gpu), _layout(v, layout, gpu)
+            last = i + 1 == len(chunks)
+            ops.attn_fwd_accumulate(qd, kd, vd, acc_o, acc_l, first=i == 0, final_out=fin if last else None)
+            bo, bl = ops.attn_fwd(qd, kd, vd)
+            ops.lse_merge(ref_o, ref_l, bo, bl, first=i == 0, final_out=ref_fin if last else None)
+            assert torch.equal(acc_o, ref_o) and torch.equal(acc_l, ref_l), (rows, i)
+            ro, rl = O.attn_fwd_ref(q, k, v)
+            oo, ol = (ro.to(dtype).double(), rl) if oo is None else O.merge_ref(oo, ol, ro.to(dtype), rl)
+        assert torch.equal(fin, ref_fin)
+        assert _err(acc_o, oo) <= 2e-2 and _err(acc_l, ol) <= 1e-3
+
+
+@pytest.mark.gpu
+def test_fused_ring_step_last_step_may_skip_the_accumulator(gpu):
+    B, H, Sq, D = 1, 2, 200, 128
+    q, k, v = (torch.randn(B, H, n, D).bfloat16().to(gpu) for n in (Sq, 300, 300))
+    acc_o = torch.randn(B, H, Sq, D, device=gpu)
+    acc_l = torch.randn(B, H, Sq, device=gpu)
+    a2, l2 = acc_o.clone(), acc_l.clone()
+    fin, fin2 = torch.empty(B, H, Sq, D, dtype=torch.bfloat16, device=gpu), torch.empty(B, H, Sq, D, dtype=torch.bfloat16, device=gpu)
+    ops.attn_fwd_accumulate(q, k, v, acc_o, acc_l, final_out=fin)
+    before = a2.clone()
+    ops.attn_fwd_accumulate(q, k, v, a2, l2, final_out=fin2, discard_acc_out=True)
+    assert torch.equal(fin, fin2) and torch.equal(acc_l, l2)
+    assert torch.equal(a2, before) and torch.equal(fin, acc_o.bfloat16())
+    with pytest.raises(ValueError):
+        ops.attn_fwd_accumulate(q, k, v, a2, l2, discard_acc_out=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("strategy", [None, "front", "rear"])
+def test_ring_loop_fused_equals_two_call_loop(gpu, monkeypatch, strategy):
+    """The BSHD ring loop takes the fused step where it can; forcing the kernel call +
+    update_out_and_lse sequence instead must give the same bits."""
+    B, S, H, D, P = 1, 4 * 300, 4, 128, 4
+    g = torch.Generator().manual_seed(9)
+    q, k, v = (torch.randn(B, S, H, D, generator=g).bfloat16().to(gpu) for _ in range(3))
+    kw = {}
+    if strategy:
+        kw = dict(joint_tensor_key=torch.randn(B, 77, H, D, generator=g).bfloat16().to(gpu),
+                  joint_tensor_value=torch.randn(B, 77, H, D, generator=g).bfloat16().to(gpu), joint_strategy=strategy)
+    o1, l1, _ = ring.xdit_ring_flash_attn_func(q, k, v, return_attn_probs=True, group=ring.LocalRing(P, rank=1), **kw)
+    monkeypatch.setattr(ops, "fused_ring_step_supported", lambda q: False)
+    o2, l2, _ = ring.xdit_ring_flash_attn_func(q, k, v, return_attn_probs=True, group=ring.LocalRing(P, rank=1), **kw)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+    kall = k if not strategy else torch.cat([k, kw["joint_tensor_key"]], 1)
+    vall = v if not strategy else torch.cat([v, kw["joint_tensor_value"]], 1)
+    ro, rl = O.attn_fwd_ref(*(t.transpose(1, 2).cpu() for t in (q, kall, vall)))
+    assert _err(o1.transpose(1, 2), ro) <= 2e-2 and _err(l1, rl) <= 1e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("strategy", [None, "front", "rear"])
+def test_usp_ring_fused_equals_merger_loop(gpu, monkeypatch, strategy):
+    """usp.ring_attn takes the fused step for our 16-bit backend (the launch count shows it); the
+    attention-function + SDPAMerger loop must give the same bits."""
+    g = torch.Generator().manual_seed(31)
+    q, k, v = (torch.randn(1, 4, 4 * 200, 128, generator=g).bfloat16().to(gpu) for _ in range(3))
+    jk = jv = None
+    mk = lambda: None
+    if strategy:
+        jk, jv = (torch.randn(1, 4, 50, 128, generator=g).bfloat16().to(gpu) for _ in range(2))
+        mk = lambda: dict(joint_key=jk, joint_value=jv, joint_strategy=strategy, step=0, total_steps=4)
+    fn = usp._get_attention_function()
+    calls = []
+    real = ops.attn_fwd_accumulate
+    monkeypatch.setattr(ops, "attn_fwd_accumulate", lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    a = usp.ring_attn(fn, q, k, v, ring_chunks=4, joint_attn_kwargs=mk())
+    assert len(calls) == 4
+    monkeypatch.setattr(ops, "fused_ring_step_supported", lambda q: False)
+    b = usp.ring_attn(fn, q, k, v, ring_chunks=4, joint_attn_kwargs=mk())
+    assert len(calls) == 4 and torch.equal(a, b)
+    kall = k if not strategy else torch.cat([jk, k] if strategy == "front" else [k, jk], 2)
+    vall = v if not strategy else torch.cat([jv, v] if strategy == "front" else [v, jv], 2)
+    ro, _ = O.attn_fwd_ref(q.cpu(), kall.cpu(), vall.cpu())
+    assert _err(a, ro) <= 2e-2
+
+
 # ---------------------------------------------------------------------------- quantiser
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_fp8_quant_bit_exact(gpu, dtype):

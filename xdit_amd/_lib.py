@@ -9,7 +9,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libxdit_amd_attn.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 XDIT_OK = 0
 XDIT_ERR_INVALID_ARG = -1
@@ -89,6 +89,19 @@ class MergeArgs(ctypes.Structure):
     ]
 
 
+class RingAcc(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("first", ctypes.c_int32),
+        ("discard_acc_out", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
+        ("acc_out", ctypes.c_void_p),
+        ("acc_lse", ctypes.c_void_p),
+        ("acc_out_stride", Strides),
+        ("acc_lse_stride", Strides),
+    ]
+
+
 class QuantArgs(ctypes.Structure):
     _fields_ = [
         ("struct_size", ctypes.c_uint32),
@@ -138,7 +151,7 @@ class PrologueArgs(ctypes.Structure):
 NORM_NONE, NORM_HEAD, NORM_TOKEN = 0, 1, 2
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_SPLIT_HALF, ROPE_WAN = 0, 1, 2, 3
 
-EXPORTS = ("xdit_attn_fwd", "xdit_attn_workspace_bytes", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_qk_prologue_batch", "xdit_attn_last_error", "xdit_attn_abi_version")
+EXPORTS = ("xdit_attn_fwd", "xdit_attn_fwd_accumulate", "xdit_attn_workspace_bytes", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_qk_prologue_batch", "xdit_attn_last_error", "xdit_attn_abi_version")
 
 _lib = None
 _lock = threading.Lock()
@@ -160,6 +173,8 @@ def lib():
         L = ctypes.CDLL(LIB_PATH)
         L.xdit_attn_fwd.argtypes = [ctypes.POINTER(AttnArgs)]
         L.xdit_attn_fwd.restype = ctypes.c_int
+        L.xdit_attn_fwd_accumulate.argtypes = [ctypes.POINTER(AttnArgs), ctypes.POINTER(RingAcc)]
+        L.xdit_attn_fwd_accumulate.restype = ctypes.c_int
         L.xdit_attn_workspace_bytes.argtypes = [ctypes.POINTER(AttnArgs)]
         L.xdit_attn_workspace_bytes.restype = ctypes.c_int64
         L.xdit_lse_merge.argtypes = [ctypes.POINTER(MergeArgs)]

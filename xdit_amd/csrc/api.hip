@@ -155,7 +155,7 @@ const char* xdit_attn_last_error(void) { return g_err; }
 
 int xdit_attn_abi_version(void) { return XDIT_ATTN_ABI_VERSION; }
 
-int xdit_attn_fwd(const xdit_attn_args* a) {
+static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   g_err[0] = 0;
   if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
   if (a->struct_size != sizeof(xdit_attn_args))
@@ -189,7 +189,20 @@ int xdit_attn_fwd(const xdit_attn_args* a) {
     if ((rc = check_tensor("k2", a->k2, a->k2_stride, es, a->D))) return rc;
     if ((rc = check_tensor("v2", a->v2, a->v2_stride, es, a->D))) return rc;
   }
-  if ((rc = check_tensor("out", a->out, a->out_stride, elem_size(out_dtype), a->D))) return rc;
+  if (acc == nullptr || a->out != nullptr)
+    if ((rc = check_tensor("out", a->out, a->out_stride, elem_size(out_dtype), a->D))) return rc;
+  if (acc != nullptr) {
+    if (acc->struct_size != sizeof(xdit_ring_acc))
+      return fail(XDIT_ERR_INVALID_ARG, "acc struct_size %u != %zu (ABI mismatch)", acc->struct_size, sizeof(xdit_ring_acc));
+    if (!((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64)))
+      return fail(XDIT_ERR_UNSUPPORTED, "the fused ring step needs bf16 or fp16 inputs with head_dim 64 or 128");
+    if ((rc = check_tensor("acc_out", acc->acc_out, acc->acc_out_stride, 4, a->D))) return rc;
+    if (acc->acc_lse == nullptr) return fail(XDIT_ERR_INVALID_ARG, "acc_lse is NULL");
+    if (acc->acc_lse_stride.b < 0 || acc->acc_lse_stride.h < 0 || acc->acc_lse_stride.s <= 0)
+      return fail(XDIT_ERR_INVALID_ARG, "acc_lse strides must be non-negative (row stride positive)");
+    if (acc->discard_acc_out != 0 && a->out == nullptr)
+      return fail(XDIT_ERR_INVALID_ARG, "discard_acc_out needs args->out to receive the result");
+  }
   if (a->lse != nullptr && (a->lse_stride_b < 0 || a->lse_stride_h < a->Sq))
     return fail(XDIT_ERR_INVALID_ARG, "lse strides (%lld,%lld) do not hold Sq=%lld rows", (long long)a->lse_stride_b, (long long)a->lse_stride_h, (long long)a->Sq);
 
@@ -208,7 +221,13 @@ int xdit_attn_fwd(const xdit_attn_args* a) {
   p.B = a->B; p.H = a->H;
   p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.scale = a->softmax_scale;
-  if (a->workspace != nullptr && a->workspace_bytes > 0 && aligned16(a->workspace)) {
+  if (acc != nullptr) {  // folded in the epilogue of whole query tiles: no shared last round
+    p.acc_out = acc->acc_out; p.acc_lse = acc->acc_lse;
+    p.ao_b = acc->acc_out_stride.b; p.ao_h = acc->acc_out_stride.h; p.ao_s = acc->acc_out_stride.s;
+    p.al_b = acc->acc_lse_stride.b; p.al_h = acc->acc_lse_stride.h; p.al_s = acc->acc_lse_stride.s;
+    p.acc_first = acc->first != 0;
+    p.acc_store = acc->discard_acc_out == 0;
+  } else if (a->workspace != nullptr && a->workspace_bytes > 0 && aligned16(a->workspace)) {
     p.ws_out = a->workspace;
     p.ws_bytes = (size_t)a->workspace_bytes;
   }
@@ -226,6 +245,16 @@ int xdit_attn_fwd(const xdit_attn_args* a) {
   }
   if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
   return XDIT_OK;
+}
+
+int xdit_attn_fwd(const xdit_attn_args* a) { return attn_fwd_impl(a, nullptr); }
+
+int xdit_attn_fwd_accumulate(const xdit_attn_args* a, const xdit_ring_acc* acc) {
+  if (acc == nullptr) {
+    g_err[0] = 0;
+    return fail(XDIT_ERR_INVALID_ARG, "acc is NULL");
+  }
+  return attn_fwd_impl(a, acc);
 }
 
 int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {

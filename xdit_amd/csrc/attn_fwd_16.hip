@@ -286,7 +286,7 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   const float l_tot = sum_halves(l_part);
   const float inv = 1.0f / l_tot;
   const float lse = (m_used * c + fast_log2(l_tot)) * kLn2;
-  if (qrow < p.Sq) {
+  if (qrow < p.Sq && (p.acc_out == nullptr || part_out != nullptr)) {
     T* optr;
     if (part_out != nullptr) optr = part_out + (wave * kRowsPerWave + l32) * D;
     else optr = (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
@@ -304,6 +304,40 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
     if (hh == 0) {
       if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
       else if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = lse;
+    }
+  } else if (qrow < p.Sq) {
+    // Ring step: fold this block into the fp32 accumulator (the arithmetic of the merge kernel
+    // on the block rounded to T, so the result equals forward + merge bit for bit).
+    float* aptr = p.acc_out + b * p.ao_b + h * p.ao_h + (int64_t)qrow * p.ao_s;
+    float* alp = p.acc_lse + b * p.al_b + h * p.al_h + (int64_t)qrow * p.al_s;
+    T* optr = p.out != nullptr ? (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s : nullptr;
+    const bool first = p.acc_first != 0;
+    float w = 0.f, new_lse = lse;
+    if (!first) {
+      const float la = *alp;
+      w = sigmoid(lse - la);
+      new_lse = la - log_sigmoid(la - lse);
+    }
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; db++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        typedef __attribute__((ext_vector_type(4))) T vec4;
+        const int d = 32 * db + 8 * a + 4 * hh;
+        f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                   oacc[db][4 * a + 3] * inv};
+        f32x4 m = __builtin_convertvector(__builtin_convertvector(o, vec4), f32x4);
+        if (!first) {
+          const f32x4 acc = *(const f32x4*)(aptr + d);
+#pragma unroll
+          for (int j = 0; j < 4; j++) m[j] = fold_value(acc[j], m[j], w);
+        }
+        if (p.acc_store) *(f32x4*)(aptr + d) = m;
+        if (optr != nullptr) *(vec4*)(optr + d) = __builtin_convertvector(m, vec4);
+      }
+    if (hh == 0) {
+      *alp = new_lse;
+      if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = new_lse;
     }
   }
 }

@@ -59,6 +59,13 @@ struct AttnParams {
   int split_share;    // KV iterations of the remaining query tiles per resident workgroup
   int split_claimers; // workgroups that process ranges
   unsigned* split_counter;  // ranges handed out beyond the first of every claimer (nullptr: one range each)
+  // ring step (optional): the result is folded into an fp32 accumulator in the epilogue
+  float* acc_out;     // (B,H,Sq,D) fp32 running output, nullptr: plain forward
+  float* acc_lse;     // (B,H,Sq) fp32 running log-sum-exp
+  int64_t ao_b, ao_h, ao_s;
+  int64_t al_b, al_h, al_s;
+  int acc_first;      // initialise the accumulator from this block instead of folding
+  int acc_store;      // write acc_out back (0: only `out` and acc_lse receive the result)
   void* ws_out;       // workspace: partial outputs [tile][slot][row][D] in the output dtype ...
   float* ws_lse;      // ... followed by partial log-sum-exps [tile][slot][row]
   size_t ws_bytes;
@@ -76,6 +83,17 @@ __device__ __forceinline__ float sum_halves(float x) {
   int xi = __builtin_bit_cast(int, x);
   auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
   return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+}
+
+// The two functions of the ring fold, shared by the merge kernel and the fused epilogue so that
+// both give the same bits.  logsigmoid(x) = min(x, 0) - log1p(exp(-|x|)), the form torch evaluates.
+__device__ __forceinline__ float log_sigmoid(float x) {
+  return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
+}
+__device__ __forceinline__ float sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+// acc - w * (acc - blk), with the rounding of one fused multiply-add.
+__device__ __forceinline__ float fold_value(float acc, float blk, float w) {
+  return __builtin_fmaf(-w, acc - blk, acc);
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

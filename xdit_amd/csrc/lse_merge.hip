@@ -56,12 +56,6 @@ template <> struct Load8<_Float16> {
   }
 };
 
-// logsigmoid(x) = min(x, 0) - log1p(exp(-|x|)), the form torch evaluates.
-__device__ __forceinline__ float log_sigmoid(float x) {
-  return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
-}
-__device__ __forceinline__ float sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
-
 template <typename TB, typename TF, bool HAS_FINAL>
 __global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p) {
   const int tpr = p.D >> 3;  // threads per row
@@ -93,7 +87,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p) {
     const float lse = *al;
     const float w = sigmoid(blse - lse);
 #pragma unroll
-    for (int i = 0; i < 8; i++) xo[i] = xo[i] - w * (xo[i] - xb[i]);
+    for (int i = 0; i < 8; i++) xo[i] = fold_value(xo[i], xb[i], w);
     new_lse = lse - log_sigmoid(lse - blse);
   }
   Load8<float>::st(ao, xo);

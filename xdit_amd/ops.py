@@ -60,7 +60,7 @@ def _workspace(device, nbytes):
 
 def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
              q_descale=None, k_descale=None, v_descale=None, out_dtype=None, out=None,
-             return_lse=True, balance=True):
+             return_lse=True, balance=True, _acc=None):
     """Non-causal attention forward on logical BHSD tensors -> (out BHSD, lse (B,H,Sq) fp32).
 
     `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
@@ -92,7 +92,8 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     if softmax_scale is None:
         softmax_scale = float(D) ** -0.5
     if out is None:
-        out = torch.empty((B, H, Sq, D), dtype=out_dtype, device=device)
+        if _acc is None:
+            out = torch.empty((B, H, Sq, D), dtype=out_dtype, device=device)
     else:
         _check4("out", out, device)
         if tuple(out.shape) != (B, H, Sq, D) or out.dtype != out_dtype:
@@ -112,8 +113,9 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     if k2 is not None and Sk2 > 0:
         a.k2, a.v2 = k2.data_ptr(), v2.data_ptr()
         a.k2_stride, a.v2_stride = _strides(k2), _strides(v2)
-    a.out = out.data_ptr()
-    a.out_stride = _strides(out)
+    if out is not None:
+        a.out = out.data_ptr()
+        a.out_stride = _strides(out)
     if lse is not None:
         a.lse = lse.data_ptr()
         a.lse_stride_b, a.lse_stride_h = lse.stride(0), lse.stride(1)
@@ -131,12 +133,47 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
         a.descale_stride_b, a.descale_stride_h = d.stride(0), d.stride(1)
     a.stream = _stream(device)
     with torch.cuda.device(device):
+        if _acc is not None:
+            _lib.check(_lib.lib().xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(_acc)))
+            return out, lse
         need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) if balance else 0
         if need > 0:
             ws = _workspace(device, need)
             a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
         _lib.check(_lib.lib().xdit_attn_fwd(ctypes.byref(a)))
     return out, lse
+
+
+def fused_ring_step_supported(q):
+    """Whether `attn_fwd_accumulate` takes these queries (bf16 / fp16, head_dim 64 or 128)."""
+    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] in (64, 128)
+
+
+def attn_fwd_accumulate(q, k, v, acc_out, acc_lse, first=False, final_out=None, discard_acc_out=False,
+                        softmax_scale=None, k2=None, v2=None):
+    """One ring step in one launch: attention of q over (k, v) [+ (k2, v2)] folded into the fp32
+    accumulator (acc_out logical BHSD, acc_lse logical BHS; any strides) exactly as `attn_fwd`
+    followed by `lse_merge` would, without the block ever reaching memory.  `first` initialises
+    the accumulator; `final_out` (logical BHSD, q's dtype) also receives the merged rows;
+    `discard_acc_out` skips the write-back of acc_out (last step).  Returns (acc_out, acc_lse)."""
+    device = q.device
+    _check4("acc_out", acc_out, device)
+    B, H, Sq, D = q.shape
+    if acc_out.dtype != torch.float32 or acc_lse.dtype != torch.float32:
+        raise ValueError("acc_out and acc_lse must be fp32")
+    if tuple(acc_out.shape) != (B, H, Sq, D) or tuple(acc_lse.shape) != (B, H, Sq) or acc_lse.device != device:
+        raise ValueError("accumulator shape mismatch")
+    if discard_acc_out and final_out is None:
+        raise ValueError("discard_acc_out needs final_out")
+    r = _lib.RingAcc()
+    r.struct_size = ctypes.sizeof(_lib.RingAcc)
+    r.first = 1 if first else 0
+    r.discard_acc_out = 1 if discard_acc_out else 0
+    r.acc_out, r.acc_lse = acc_out.data_ptr(), acc_lse.data_ptr()
+    r.acc_out_stride = _strides(acc_out)
+    r.acc_lse_stride = _lib.Strides(acc_lse.stride(0), acc_lse.stride(1), acc_lse.stride(2))
+    attn_fwd(q, k, v, softmax_scale=softmax_scale, k2=k2, v2=v2, out=final_out, return_lse=False, _acc=r)
+    return acc_out, acc_lse
 
 
 def lse_merge(acc_out, acc_lse, block_out, block_lse, first=False, final_out=None):

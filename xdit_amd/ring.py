@@ -124,6 +124,10 @@ def xdit_ring_flash_attn_forward(process_group, q, k, v, softmax_scale, dropout_
     out = None
     lse = None
     final = None
+    # bf16 / fp16 at head_dim 64 or 128: every step is one launch that folds its block into the
+    # accumulator in the kernel's epilogue (same bits as kernel call + update_out_and_lse).
+    fused = P > 1 and ops.fused_ring_step_supported(q)
+    t = lambda x: None if x is None else x.transpose(1, 2)
     for step, c in enumerate(process_group.order()):
         key, value = k_chunks[c], v_chunks[c]
         jk = jv = None
@@ -132,6 +136,19 @@ def xdit_ring_flash_attn_forward(process_group, q, k, v, softmax_scale, dropout_
                 jk, jv = joint_tensor_key, joint_tensor_value
             else:  # "front": the joint tokens come first
                 key, value, jk, jv = joint_tensor_key, joint_tensor_value, key, value
+        if fused:
+            _check_kernel_options(dropout_p, causal and step == 0, window_size, 0.0, alibi_slopes)
+            B, Sq, H, D = q.shape
+            if out is None:
+                out = torch.empty((B, Sq, H, D), dtype=torch.float32, device=q.device)
+                lse = torch.empty((B, Sq, H, 1), dtype=torch.float32, device=q.device)
+            last = step + 1 == P
+            if last:
+                final = torch.empty((B, Sq, H, D), dtype=out_dtype, device=q.device)
+            ops.attn_fwd_accumulate(t(q), t(key), t(value), t(out), lse.squeeze(-1).transpose(1, 2), first=step == 0,
+                                    final_out=t(final), discard_acc_out=last, softmax_scale=softmax_scale,
+                                    k2=t(jk), v2=t(jv))
+            continue
         block_out, block_lse = flash_attn_forward(
             q, key, value, dropout_p=dropout_p, softmax_scale=softmax_scale, causal=causal and step == 0,
             window_size=window_size, softcap=0.0, alibi_slopes=alibi_slopes, return_softmax=False,

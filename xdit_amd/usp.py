@@ -12,6 +12,7 @@ import functools
 import torch
 
 from . import ops
+from . import attention_backend as AB
 from .attention_backend import ATTENTION_FUNCTION_REGISTRY, AttentionBackendType
 
 _DEFAULT_BACKEND = AttentionBackendType.MI355
@@ -118,6 +119,30 @@ def ring_attn(attention_function, query, key, value, dropout_p=0.0, is_causal=Fa
         order = [0] + list(range(P - 1, 0, -1))
     k_chunks = key.chunk(P, dim=2)
     v_chunks = value.chunk(P, dim=2)
+    base = getattr(attention_function, "__wrapped__", attention_function)
+    if (P > 1 and ops.fused_ring_step_supported(query) and not torch.compiler.is_compiling()
+            and base is ATTENTION_FUNCTION_REGISTRY.get(AttentionBackendType.MI355)):
+        # every step is one launch: the kernel folds its block into the accumulator itself (same
+        # bits as the call + merge below); the joint keys/values join on the step the decorator
+        # would pick
+        AB._check_call(dropout_p, is_causal, attention_kwargs)
+        acc_out = torch.empty(query.shape, dtype=torch.float32, device=query.device)
+        acc_lse = torch.empty(query.shape[:3], dtype=torch.float32, device=query.device)
+        final = torch.empty(query.shape, dtype=query.dtype, device=query.device)
+        for i, c in enumerate(order):
+            joint_kv = None
+            if joint_attn_kwargs is not None:
+                strategy = joint_attn_kwargs.get("joint_strategy", None)
+                step = joint_attn_kwargs.get("step", 0)
+                if (strategy == "front" and step == 0) or (strategy == "rear" and step == joint_attn_kwargs.get("total_steps", 1) - 1):
+                    joint_kv = (joint_attn_kwargs.get("joint_key", None), joint_attn_kwargs.get("joint_value", None), strategy)
+                joint_attn_kwargs["step"] = step + 1
+            k1, v1, k2, v2 = AB._split_joint(k_chunks[c], v_chunks[c], joint_kv)
+            last = i == P - 1
+            ops.attn_fwd_accumulate(query, k1, v1, acc_out, acc_lse, first=i == 0,
+                                    final_out=final if last else None, discard_acc_out=last,
+                                    softmax_scale=query.shape[-1] ** -0.5, k2=k2, v2=v2)
+        return final
     merger = SDPAMerger()
     for i, c in enumerate(order):
         out, lse = attention_function(query, k_chunks[c], v_chunks[c], dropout_p=dropout_p, is_causal=is_causal,
