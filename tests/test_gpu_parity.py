@@ -134,15 +134,17 @@ def force_rows(monkeypatch):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind", ["bf16", "fp8"])
-def test_claimed_ranges_vs_plain_launch_and_fp32(gpu, force_rows, kind):
-    """384 query tiles of 384 rows over 256 KV iterations: the 128 tiles of the second round are
-    cut into 512 ranges of 64 iterations which the 256 workgroups of the bf16 kernel claim from a
-    counter (the fp8 kernel gives every workgroup one range of 128).  The result must match the
+@pytest.mark.parametrize("kind,rows,Sk", [("bf16", 384, 256 * 64), ("bf16", 256, 512 * 64), ("bf16", 128, 512 * 64),
+                                          ("fp8", 384, 256 * 64)])
+def test_claimed_ranges_vs_plain_launch_and_fp32(gpu, force_rows, kind, rows, Sk):
+    """Query tiles that leave a long share of KV iterations per workgroup in the last round (at 384
+    rows: 384 tiles, 128 of them shared, 128 iterations per workgroup): the bf16 kernel cuts the
+    shares into ranges of 64 iterations which the workgroups claim from a counter, at every
+    workgroup shape (the fp8 kernel gives every workgroup one range).  The result must match the
     plain launch, a fp32 computation of two heads, and itself on a second call (which workgroup
     takes which range changes nothing)."""
-    force_rows(384)
-    B, H, Sq, Sk = 1, 12, 32 * 384, 256 * 64
+    force_rows(rows)
+    B, H, Sq = 1, 12, 32 * 384
     g = torch.Generator(device=gpu).manual_seed(77)
     q, k, v = (torch.randn(B, H, n, 128, generator=g, device=gpu) for n in (Sq, Sk, Sk))
     if kind == "fp8":
