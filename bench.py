@@ -32,7 +32,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-MEASURED_HBM_BYTES_PER_LAUNCH = 210.3e6  # Flux-1024 bf16 step: 152.8 MB read + 57.5 MB written (attention + combine kernels)
+MEASURED_HBM_BYTES_PER_LAUNCH = 201.6e6  # Flux-1024 bf16 step: 147.3 MB read + 54.3 MB written (attention + combine kernels)
 
 
 def make_inputs(B, H, S, D, seed, device, rmsnorm=True, dtype=torch.bfloat16):
