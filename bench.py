@@ -203,7 +203,13 @@ def main():
         mbytes = 10.0 * N * D + 12.0 * N
         also["lse_merge_fold"] = {"us": round(ms * 1e3, 2), "gbs": round(mbytes / ms / 1e6, 1),
                                   "frac_hbm_peak": round(mbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": mbytes}
-        del acc, qb, kb, vb
+        # the last fold of a two-call ring, with the cast to bf16 fused: 12*N*D + 12*N bytes
+        fin = torch.empty_like(q)
+        _, ms = time_calls(lambda: ops.lse_merge(acc, acc_l, q, blk_l, final_out=fin), max(20, n), 5)
+        fbytes = 12.0 * N * D + 12.0 * N
+        also["lse_merge_fold_with_cast"] = {"us": round(ms * 1e3, 2), "gbs": round(fbytes / ms / 1e6, 1),
+                                            "frac_hbm_peak": round(fbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": fbytes}
+        del acc, qb, kb, vb, fin
         # HunyuanVideo 720p one-GPU head shard
         Bh, Hh, Sh = 1, 3, 118800 + 256
         qh, kh, vh = make_inputs(Bh, Hh, Sh, D, 1004, dev)
