@@ -109,6 +109,36 @@ int xdit_attn_fwd(const xdit_attn_args* args);
 int64_t xdit_attn_workspace_bytes(const xdit_attn_args* args);
 
 /*
+ * How xdit_attn_fwd would launch this problem when given the workspace it asks for (pointers of
+ * `args` are not inspected): for tests, tuning and capacity planning.  The query rows are cut
+ * into `query_tiles` tiles of `rows_per_workgroup` rows, each with `kv_iterations` tiles of 64
+ * keys.  `whole_tiles` of them are run by one workgroup each; with ranges > 0 the KV iterations
+ * of the other tiles, laid end to end, are cut into `ranges` ranges of `range_len` iterations
+ * (the last one shorter) that go to `claimers` workgroups: workgroup ids first_claimer ..
+ * first_claimer + claimers - 1, of which those below whole_tiles run a whole tile first; claimer
+ * c starts with range c and, with counter != 0, takes further ranges from a counter in the
+ * workspace.  A query tile's partial results occupy at most `slots_per_tile` workspace slots.
+ * bf16 / fp16 (head_dim 64, 128) and fp8 (head_dim 128) only.  No counterpart in the reference.
+ */
+typedef struct {
+  uint32_t struct_size;        /* = sizeof(xdit_launch_plan), set by the caller */
+  int32_t rows_per_workgroup;
+  int32_t query_tiles;
+  int32_t kv_iterations;
+  int64_t workspace_bytes;     /* = xdit_attn_workspace_bytes(args) */
+  int32_t whole_tiles;
+  int32_t ranges;
+  int32_t range_len;
+  int32_t slots_per_tile;
+  int32_t claimers;
+  int32_t first_claimer;
+  int32_t counter;
+  int32_t workgroups;          /* grid of the attention kernel */
+} xdit_launch_plan;
+
+int xdit_attn_launch_plan(const xdit_attn_args* args, xdit_launch_plan* plan);
+
+/*
  * One fold of the ring online-softmax merge, in fp32:
  *     acc_out <- acc_out - sigmoid(block_lse - acc_lse) * (acc_out - block_out)
  *     acc_lse <- acc_lse - logsigmoid(acc_lse - block_lse)

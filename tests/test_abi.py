@@ -233,3 +233,90 @@ def test_fused_ring_step_rejects_bad_arguments():
     r.discard_acc_out = 1
     a.out = 0
     assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "discard_acc_out" in _lib.last_error()
+
+
+def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128):
+    a = _attn_args(B=B, H=H, Sq=Sq, Sk=Sk, Sk2=Sk2, D=D)
+    if dtype is not None:
+        a.dtype = dtype
+        a.out_dtype = _lib.DTYPE_BF16
+    if Sk2:
+        a.k2 = a.v2 = 0x1000
+    p = _lib.LaunchPlan()
+    p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
+    rc = _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p))
+    assert rc == 0, _lib.last_error()
+    assert p.workspace_bytes == _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
+    return p
+
+
+def test_launch_plan_invariants(monkeypatch):
+    """The launch geometry for a few hundred random problems: the ranges partition the KV iterations
+    of the shared query tiles exactly, every part of a tile has a workspace slot of its own below
+    slots_per_tile, the claimers fit the grid, and the workspace holds all slots (host arithmetic
+    only; 256 compute units are assumed without a GPU)."""
+    import random
+    rng = random.Random(1234)
+    seen_counter = seen_fused = seen_separate = seen_plain = 0
+    for trial in range(400):
+        rows_env = rng.choice([None, "128", "256", "384"])
+        if rows_env is None:
+            monkeypatch.delenv("XDIT_ATTN_ROWS", raising=False)
+        else:
+            monkeypatch.setenv("XDIT_ATTN_ROWS", rows_env)
+        fp8 = rng.random() < 0.25
+        B, H = rng.choice([1, 1, 2]), rng.choice([1, 3, 5, 12, 24, 40, 64])
+        Sq = rng.choice([rng.randint(1, 4000), rng.randint(4000, 40000), rng.randint(40000, 130000)])
+        Sk = rng.choice([rng.randint(1, 600), rng.randint(600, 20000), rng.randint(20000, 130000)])
+        Sk2 = rng.choice([0, 0, rng.randint(1, 600)])
+        p = _plan(B, H, Sq, Sk, Sk2, dtype=_lib.DTYPE_FP8_E4M3FN if fp8 else None)
+        rows, nt = p.rows_per_workgroup, p.kv_iterations
+        assert rows in (128, 256, 384) and (rows_env is None or rows == int(rows_env))
+        assert p.query_tiles == B * H * -(-Sq // rows) and nt == -(-Sk // 64) + -(-Sk2 // 64)
+        if p.ranges == 0:
+            seen_plain += 1
+            assert p.workspace_bytes == 0 and p.whole_tiles == p.query_tiles and p.claimers == 0 and p.counter == 0
+            assert p.workgroups >= p.query_tiles and p.workgroups % 8 == 0
+            continue
+        rem = p.query_tiles - p.whole_tiles
+        work = rem * nt
+        assert 0 < rem and p.range_len >= 1
+        assert (p.ranges - 1) * p.range_len < work <= p.ranges * p.range_len          # exact partition
+        assert 1 <= p.claimers <= p.ranges and (p.counter == 1) == (p.ranges > p.claimers)
+        assert not fp8 or p.counter == 0
+        if p.first_claimer + p.claimers <= p.whole_tiles:                              # claimers are whole-tile workgroups
+            seen_fused += 1
+            assert p.workgroups == p.whole_tiles and p.first_claimer == p.whole_tiles - p.claimers
+        else:
+            seen_separate += 1
+            assert p.first_claimer == p.whole_tiles and p.workgroups == p.whole_tiles + p.claimers
+        seen_counter += p.counter
+        # slots: the parts of shared tile r are the ranges that intersect [r nt, (r+1) nt)
+        for r in {0, rem - 1, rng.randrange(rem)}:
+            first = (r * nt) // p.range_len
+            last = ((r + 1) * nt - 1) // p.range_len
+            assert last < p.ranges and last - first + 1 <= p.slots_per_tile
+        parts = rem * p.slots_per_tile * rows * (128 * 2 + 4)
+        assert p.workspace_bytes == (((parts + 255) & ~255) + 256 if p.counter else parts)
+    assert seen_counter > 10 and seen_fused > 10 and seen_plain > 10
+
+
+def test_launch_plan_of_the_named_shapes(monkeypatch):
+    monkeypatch.delenv("XDIT_ATTN_ROWS", raising=False)
+    flux = _plan(1, 24, 4608, 4608)
+    assert (flux.rows_per_workgroup, flux.query_tiles, flux.whole_tiles, flux.ranges, flux.range_len,
+            flux.claimers, flux.first_claimer, flux.counter, flux.workgroups) == (384, 288, 256, 256, 9, 256, 0, 0, 256)
+    hv = _plan(1, 3, 118800 + 256, 118800 + 256)
+    assert (hv.rows_per_workgroup, hv.query_tiles, hv.whole_tiles, hv.kv_iterations) == (384, 933, 768, 1861)
+    assert (hv.ranges, hv.range_len, hv.claimers, hv.first_claimer, hv.counter, hv.workgroups) == (1536, 200, 256, 512, 1, 768)
+    wan = _plan(1, 5, 75600, 75600, dtype=_lib.DTYPE_FP8_E4M3FN)
+    assert (wan.rows_per_workgroup, wan.whole_tiles, wan.ranges, wan.claimers, wan.counter) == (384, 768, 256, 256, 0)
+    ring_chunk = _plan(1, 24, 4608, 1152)
+    assert (ring_chunk.rows_per_workgroup, ring_chunk.ranges, ring_chunk.workgroups) == (256, 0, 432)
+    p = _lib.LaunchPlan()
+    p.struct_size = 4
+    a = _attn_args()
+    assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == _lib.XDIT_ERR_INVALID_ARG
+    p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
+    a.dtype = a.out_dtype = _lib.DTYPE_FP32
+    assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == _lib.XDIT_ERR_UNSUPPORTED

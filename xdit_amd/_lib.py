@@ -89,6 +89,24 @@ class MergeArgs(ctypes.Structure):
     ]
 
 
+class LaunchPlan(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("rows_per_workgroup", ctypes.c_int32),
+        ("query_tiles", ctypes.c_int32),
+        ("kv_iterations", ctypes.c_int32),
+        ("workspace_bytes", ctypes.c_int64),
+        ("whole_tiles", ctypes.c_int32),
+        ("ranges", ctypes.c_int32),
+        ("range_len", ctypes.c_int32),
+        ("slots_per_tile", ctypes.c_int32),
+        ("claimers", ctypes.c_int32),
+        ("first_claimer", ctypes.c_int32),
+        ("counter", ctypes.c_int32),
+        ("workgroups", ctypes.c_int32),
+    ]
+
+
 class RingAcc(ctypes.Structure):
     _fields_ = [
         ("struct_size", ctypes.c_uint32),
@@ -151,7 +169,7 @@ class PrologueArgs(ctypes.Structure):
 NORM_NONE, NORM_HEAD, NORM_TOKEN = 0, 1, 2
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_SPLIT_HALF, ROPE_WAN = 0, 1, 2, 3
 
-EXPORTS = ("xdit_attn_fwd", "xdit_attn_fwd_accumulate", "xdit_attn_workspace_bytes", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_qk_prologue_batch", "xdit_attn_last_error", "xdit_attn_abi_version")
+EXPORTS = ("xdit_attn_fwd", "xdit_attn_fwd_accumulate", "xdit_attn_workspace_bytes", "xdit_attn_launch_plan", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_qk_prologue_batch", "xdit_attn_last_error", "xdit_attn_abi_version")
 
 _lib = None
 _lock = threading.Lock()
@@ -175,6 +193,8 @@ def lib():
         L.xdit_attn_fwd.restype = ctypes.c_int
         L.xdit_attn_fwd_accumulate.argtypes = [ctypes.POINTER(AttnArgs), ctypes.POINTER(RingAcc)]
         L.xdit_attn_fwd_accumulate.restype = ctypes.c_int
+        L.xdit_attn_launch_plan.argtypes = [ctypes.POINTER(AttnArgs), ctypes.POINTER(LaunchPlan)]
+        L.xdit_attn_launch_plan.restype = ctypes.c_int
         L.xdit_attn_workspace_bytes.argtypes = [ctypes.POINTER(AttnArgs)]
         L.xdit_attn_workspace_bytes.restype = ctypes.c_int64
         L.xdit_lse_merge.argtypes = [ctypes.POINTER(MergeArgs)]

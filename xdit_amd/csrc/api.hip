@@ -273,6 +273,42 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
   return (int64_t)xdit::attn_fwd_16_workspace(p, a->D, rows_per_block_16(a));
 }
 
+int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
+  g_err[0] = 0;
+  if (a == nullptr || out == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args or plan is NULL");
+  if (a->struct_size != sizeof(xdit_attn_args))
+    return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_attn_args));
+  if (out->struct_size != sizeof(xdit_launch_plan))
+    return fail(XDIT_ERR_INVALID_ARG, "plan struct_size %u != %zu (ABI mismatch)", out->struct_size, sizeof(xdit_launch_plan));
+  if (a->B <= 0 || a->H <= 0 || a->Sq <= 0 || a->Sk <= 0 || a->Sk2 < 0 || a->Sq > (int64_t(1) << 30) ||
+      a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30))
+    return fail(XDIT_ERR_INVALID_ARG, "bad shape");
+  const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128;
+  const bool b16 = (a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64);
+  if (!fp8 && !b16) return fail(XDIT_ERR_UNSUPPORTED, "no launch plan for this dtype / head_dim (generic kernel: one workgroup per 64 query rows)");
+  xdit::AttnParams p, q;
+  std::memset(&p, 0, sizeof(p));
+  p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
+  const int rows = rows_per_block_16(a);
+  const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q) : xdit::attn_fwd_16_workspace(p, a->D, rows, &q);
+  const uint32_t size = out->struct_size;
+  std::memset(out, 0, sizeof(*out));
+  out->struct_size = size;
+  out->rows_per_workgroup = rows;
+  out->query_tiles = q.total_tiles;
+  out->kv_iterations = (int32_t)((a->Sk + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile + (a->Sk2 + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile);
+  out->workspace_bytes = (int64_t)need;
+  out->whole_tiles = q.split_units ? q.split_full : q.total_tiles;
+  out->ranges = q.split_units;
+  out->range_len = q.split_len;
+  out->slots_per_tile = q.split_pmax;
+  out->claimers = q.split_claimers;
+  out->first_claimer = q.split_units ? (q.split_fuse0 <= q.split_full ? q.split_fuse0 : q.split_full) : 0;
+  out->counter = q.split_units > q.split_claimers ? 1 : 0;
+  out->workgroups = (int32_t)xdit::split_grid(q);
+  return XDIT_OK;
+}
+
 int xdit_lse_merge(const xdit_merge_args* a) {
   g_err[0] = 0;
   if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");

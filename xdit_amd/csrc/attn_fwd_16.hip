@@ -379,21 +379,25 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_
   return hipGetLastError();
 }
 
-// Workspace bytes a balanced launch of this problem would use (0: none needed).
+// Workspace bytes a balanced launch of this problem would use (0: none needed); `plan`, if given,
+// receives the launch geometry (as if that workspace were supplied).
 template <int D, int NW>
-static size_t workspace_one(const AttnParams& p) {
+static size_t workspace_one(const AttnParams& p, AttnParams* plan) {
   AttnParams q = p;
   constexpr int rows = 32 * NW;
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
-  return plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup);
+  q.tiles_per_xcd = (q.total_tiles + 7) / 8;
+  const size_t need = plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup);
+  if (plan != nullptr) *plan = q;
+  return need;
 }
 
-size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block) {
-  if (D == 128 && rows_per_block == 384) return workspace_one<128, 12>(p);
-  if (D == 128 && rows_per_block == 256) return workspace_one<128, 8>(p);
-  if (D == 128) return workspace_one<128, 4>(p);
-  if (D == 64) return workspace_one<64, 4>(p);
+size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block, AttnParams* plan) {
+  if (D == 128 && rows_per_block == 384) return workspace_one<128, 12>(p, plan);
+  if (D == 128 && rows_per_block == 256) return workspace_one<128, 8>(p, plan);
+  if (D == 128) return workspace_one<128, 4>(p, plan);
+  if (D == 64) return workspace_one<64, 4>(p, plan);
   return 0;
 }
 

@@ -341,12 +341,15 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
 }
 
 template <int NW>
-static size_t workspace_one(const AttnParams& p) {
+static size_t workspace_one(const AttnParams& p, AttnParams* plan) {
   AttnParams q = p;
   constexpr int rows = kRowsPerWave * NW;
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
-  return plan_split(q, rows, resident_workgroups(NW), D, 2, 1);
+  q.tiles_per_xcd = (q.total_tiles + 7) / 8;
+  const size_t need = plan_split(q, rows, resident_workgroups(NW), D, 2, 1);
+  if (plan != nullptr) *plan = q;
+  return need;
 }
 
 }  // namespace fp8path
@@ -359,11 +362,11 @@ hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_pe
   return out_is_fp16 ? launch_one<_Float16, 4>(p, stream) : launch_one<__bf16, 4>(p, stream);
 }
 
-size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block) {
+size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan) {
   using namespace fp8path;
-  if (rows_per_block == 384) return workspace_one<12>(p);
-  if (rows_per_block == 256) return workspace_one<8>(p);
-  return workspace_one<4>(p);
+  if (rows_per_block == 384) return workspace_one<12>(p, plan);
+  if (rows_per_block == 256) return workspace_one<8>(p, plan);
+  return workspace_one<4>(p, plan);
 }
 
 }  // namespace xdit
