@@ -157,6 +157,8 @@ def test_claimed_ranges_vs_plain_launch_and_fp32(gpu, force_rows, kind, rows, Sk
         args, kw = tuple(t.to(torch.bfloat16) for t in (q, k, v)), {}
         qf, kf, vf = (t.float() for t in args)
         tol_o, tol_l = TOL[torch.bfloat16]
+    plan = ops.launch_plan(args[0], args[1])
+    assert plan["rows_per_workgroup"] == rows and plan["ranges"] > 0 and plan["counter"] == (kind == "bf16")
     o, l = ops.attn_fwd(*args, **kw)
     o1, l1 = ops.attn_fwd(*args, balance=False, **kw)
     assert (o.float() - o1.float()).abs().max().item() <= 1e-2 and (l - l1).abs().max().item() <= 1e-5

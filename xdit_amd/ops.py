@@ -144,6 +144,24 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     return out, lse
 
 
+def launch_plan(q, k, k2=None):
+    """How `attn_fwd(q, k, v, k2=..)` would be launched (a dict of the fields of xdit_launch_plan):
+    rows per workgroup, query tiles, whole tiles, shared ranges and their length, claimers,
+    whether ranges are handed out through the counter, workgroups, workspace bytes.  Host
+    arithmetic only; bf16 / fp16 (head_dim 64, 128) and fp8 (head_dim 128)."""
+    a = _lib.AttnArgs()
+    a.struct_size = ctypes.sizeof(_lib.AttnArgs)
+    a.dtype = _code(q.dtype)
+    a.out_dtype = _code(torch.bfloat16 if q.dtype == torch.float8_e4m3fn else q.dtype)
+    a.B, a.H, a.Sq, a.D = q.shape
+    a.Sk = k.shape[2]
+    a.Sk2 = 0 if k2 is None else k2.shape[2]
+    p = _lib.LaunchPlan()
+    p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
+    _lib.check(_lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)))
+    return {name: getattr(p, name) for name, _ in _lib.LaunchPlan._fields_ if name != "struct_size"}
+
+
 def fused_ring_step_supported(q):
     """Whether `attn_fwd_accumulate` takes these queries (bf16 / fp16, head_dim 64 or 128)."""
     return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] in (64, 128)
