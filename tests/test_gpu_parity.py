@@ -172,7 +172,7 @@ def test_claimed_ranges_vs_plain_launch_and_fp32(gpu, force_rows, kind, rows, Sk
 
 
 @pytest.mark.parametrize("rows", [128, 256, 384])
-@pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8"])
+@pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8", "bf16-d64", "fp16-d64"])
 @pytest.mark.parametrize("B,H,Sq,Sk,Sk2", [
     (1, 2, 1000, 777, 0),       # several workgroups per head, partial last query tile and KV tile
     (1, 1, 385, 8192, 0),       # balanced launch: KV ranges shared between workgroups
@@ -180,11 +180,13 @@ def test_claimed_ranges_vs_plain_launch_and_fp32(gpu, force_rows, kind, rows, Sk
     (2, 2, 50, 64, 1),          # fewer query rows than one workgroup covers
 ])
 def test_workgroup_shapes_vs_oracle(gpu, force_rows, rows, kind, B, H, Sq, Sk, Sk2):
-    """Every workgroup shape of the 16-bit and fp8 kernels, with and without the balanced launch,
-    against the oracle on the same inputs."""
+    """Every workgroup shape of the 16-bit (head_dim 128 and 64) and fp8 kernels, with and without
+    the balanced launch, against the oracle on the same inputs."""
     force_rows(rows)
+    D = 64 if kind.endswith("-d64") else 128
+    kind = kind.split("-")[0]
     g = torch.Generator().manual_seed(rows + Sq + Sk)
-    mk = lambda n: torch.randn(B, H, n, 128, generator=g)
+    mk = lambda n: torch.randn(B, H, n, D, generator=g)
     q, k, v = mk(Sq), mk(Sk), mk(Sk)
     k2, v2 = (mk(Sk2), mk(Sk2)) if Sk2 else (None, None)
     dev = lambda t: None if t is None else t.to(gpu)
@@ -211,6 +213,7 @@ def test_workgroup_shapes_vs_oracle(gpu, force_rows, rows, kind, B, H, Sq, Sk, S
         ro, rl = O.attn_fwd_ref(q, kall, vall)
         args = (dev(q), dev(k), dev(v))
         tol_o, tol_l = TOL[dt]
+    assert ops.launch_plan(args[0], args[1], k2=kw.get("k2"))["rows_per_workgroup"] == rows
     o, l = ops.attn_fwd(*args, **kw)
     o1, l1 = ops.attn_fwd(*args, balance=False, **kw)
     assert _err(o, ro) <= tol_o and _err(l, rl) <= tol_l

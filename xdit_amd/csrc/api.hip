@@ -52,15 +52,15 @@ int check_tensor(const char* name, const void* p, const xdit_strides& st, int es
   return 0;
 }
 
-// Query rows per workgroup (head_dim 128: 384, 256 or 128, i.e. 12, 8 or 4 wavefronts sharing each
-// K/V tile).  Picks the shape with the shortest estimated critical path: KV iterations of the
+// Query rows per workgroup (head_dim 128 and 64: 384, 256 or 128, i.e. 12, 8 or 4 wavefronts
+// sharing each K/V tile; other head_dims: 128).  Picks the shape with the shortest estimated critical path: KV iterations of the
 // busiest compute unit (whole rounds of resident workgroups, or the balanced launch's shared last
 // round plus its fixed cost) times the rows a compute unit works on per iteration, with a small
 // penalty for the shapes that share a tile between fewer wavefronts.  Measured on Flux-1024
 // (72 KV tiles: 384 rows wins through the balanced launch) and on its ring chunks (18 KV tiles:
 // 256 rows, 0.079 ms against 0.101 ms at 384).
 int rows_per_block_16(const xdit_attn_args* a) {
-  if (a->D != 128) return 128;
+  if (a->D != 128 && a->D != 64) return 128;
   const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128", "256" or "384": testing aid, read per call
   if (force != nullptr) {
     const int r = std::atoi(force);
@@ -71,7 +71,12 @@ int rows_per_block_16(const xdit_attn_args* a) {
   const int64_t bh = (int64_t)a->B * a->H;
   const int64_t nt = (a->Sk + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile + (a->Sk2 + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile;
   static const int kRows[3] = {384, 256, 128};
-  static const double kPenalty[3] = {1.0, 1.06, 1.12};
+  // head_dim 64: 384 and 128 rows run at the same rate, 256 rows 5 % slower (B=1 H=48 S=17776:
+  // 4.21 / 4.41 / 4.15 ms at 384 / 256 / 128 rows; a 1063-key ring chunk of B=2 H=24 S=4250:
+  // 103 / 96 / 79 us), so the number of rounds decides
+  static const double kPenalty128[3] = {1.0, 1.06, 1.12};
+  static const double kPenalty64[3] = {1.0, 1.10, 1.0};
+  const double* kPenalty = a->D == 64 ? kPenalty64 : kPenalty128;
   int best = 128;
   double best_cost = 0;
   for (int i = 0; i < 3; i++) {
@@ -83,9 +88,12 @@ int rows_per_block_16(const xdit_attn_args* a) {
     xdit::AttnParams q;
     std::memset(&q, 0, sizeof(q));
     q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
-    xdit::plan_split(q, rows, slots, 128, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup);
-    const double units = q.split_units ? (double)(q.split_full / slots) * nt + q.split_share + 10
-                                       : (double)((tiles + slots - 1) / slots) * nt;
+    xdit::plan_split(q, rows, slots, a->D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup);
+    // every segment costs a few iterations' worth of prologue and epilogue (about 13 us: 5
+    // iterations at head_dim 128, 9 at head_dim 64), the combine pass about as much again
+    const double ovh = a->D == 64 ? 9.0 : 5.0;
+    const double units = q.split_units ? (double)(q.split_full / slots) * (nt + ovh) + q.split_share + 2 * ovh
+                                       : (double)((tiles + slots - 1) / slots) * (nt + ovh);
     int64_t sharing = (tiles + cus - 1) / cus;  // workgroups on the busiest compute unit at once
     if (sharing > per_cu) sharing = per_cu;
     const double cost = units * rows * (double)sharing * kPenalty[i];

@@ -397,21 +397,26 @@ size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block, Att
   if (D == 128 && rows_per_block == 384) return workspace_one<128, 12>(p, plan);
   if (D == 128 && rows_per_block == 256) return workspace_one<128, 8>(p, plan);
   if (D == 128) return workspace_one<128, 4>(p, plan);
+  if (D == 64 && rows_per_block == 384) return workspace_one<64, 12>(p, plan);
+  if (D == 64 && rows_per_block == 256) return workspace_one<64, 8>(p, plan);
   if (D == 64) return workspace_one<64, 4>(p, plan);
   return 0;
 }
 
 // Host-side launcher (called from the C ABI after argument validation).
-// rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12 wavefronts); the larger two are for
-// head_dim 128 only.
+// rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12 wavefronts), for head_dim 128 and 64.
 hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream) {
-  static bool ready[8] = {false, false, false, false, false, false, false, false};
+  static bool ready[12] = {false, false, false, false, false, false, false, false, false, false, false, false};
   if (D == 128 && rows_per_block == 384) {
     return dtype_is_fp16 ? launch_one<_Float16, 128, 12>(p, stream, ready[6]) : launch_one<__bf16, 128, 12>(p, stream, ready[7]);
   } else if (D == 128 && rows_per_block == 256) {
     return dtype_is_fp16 ? launch_one<_Float16, 128, 8>(p, stream, ready[4]) : launch_one<__bf16, 128, 8>(p, stream, ready[5]);
   } else if (D == 128) {
     return dtype_is_fp16 ? launch_one<_Float16, 128, 4>(p, stream, ready[0]) : launch_one<__bf16, 128, 4>(p, stream, ready[1]);
+  } else if (D == 64 && rows_per_block == 384) {
+    return dtype_is_fp16 ? launch_one<_Float16, 64, 12>(p, stream, ready[10]) : launch_one<__bf16, 64, 12>(p, stream, ready[11]);
+  } else if (D == 64 && rows_per_block == 256) {
+    return dtype_is_fp16 ? launch_one<_Float16, 64, 8>(p, stream, ready[8]) : launch_one<__bf16, 64, 8>(p, stream, ready[9]);
   } else if (D == 64) {
     return dtype_is_fp16 ? launch_one<_Float16, 64, 4>(p, stream, ready[2]) : launch_one<__bf16, 64, 4>(p, stream, ready[3]);
   }
