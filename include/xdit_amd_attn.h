@@ -62,6 +62,9 @@ typedef struct {
  *     s_ij = softmax_scale * sum_d q_id k_jd ,  j over Sk keys of (k,v) then Sk2 keys of (k2,v2)
  *     out_i = sum_j softmax_j(s_ij) v_j ,  lse_i = log sum_j exp(s_ij)
  * For FP8 inputs q,k,v are multiplied by q_descale[b,h], k_descale[b,h], v_descale[b,h] first.
+ * head_dim: a multiple of 8; bf16 / fp16 / fp32 up to 128 (bf16 and fp16 on the 16-bit matrix
+ * cores at every such head_dim, at the cost of the next of 64 / 128; fp32 on the fp32 matrix
+ * cores), fp8 exactly 128.
  * Replaces: attention_backend.py:504-516/:774-823/:887-918 (+ :617-642, :717-772 for fp8) and the
  * kernel call at ring_flash_attn.py:123-134.  The optional second KV segment replaces the
  * torch.cat of joint (text) keys/values at usp.py:239-241 / ring_flash_attn.py:89-100.
@@ -118,7 +121,8 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* args);
  * first_claimer + claimers - 1, of which those below whole_tiles run a whole tile first; claimer
  * c starts with range c and, with counter != 0, takes further ranges from a counter in the
  * workspace.  A query tile's partial results occupy at most `slots_per_tile` workspace slots.
- * bf16 / fp16 (head_dim 64, 128) and fp8 (head_dim 128) only.  No counterpart in the reference.
+ * bf16 / fp16 (head_dim up to 128; the geometry is that of head_dim 64 or 128, whichever is
+ * the next one up) and fp8 (head_dim 128) only.  No counterpart in the reference.
  */
 typedef struct {
   uint32_t struct_size;        /* = sizeof(xdit_launch_plan), set by the caller */
@@ -183,8 +187,8 @@ int xdit_lse_merge(const xdit_merge_args* args);
  *                         carry the result); needs args->out
  * acc_out is logical (B,H,Sq,D) fp32, acc_lse logical (B,H,Sq) fp32 with its own strides (the
  * (B,S,H,1) accumulator of the legacy ring maps without a copy).  bf16 / fp16 inputs with
- * head_dim 64 or 128; XDIT_ERR_UNSUPPORTED otherwise (use the two calls).  args->workspace is
- * not used.
+ * head_dim a multiple of 8 up to 128; XDIT_ERR_UNSUPPORTED otherwise (use the two calls).
+ * args->workspace is not used.
  * Replaces, per ring step: the kernel call at ring_flash_attn.py:123-134, update_out_and_lse at
  * :138 and, on the last step, the cast at :145.
  */

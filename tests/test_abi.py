@@ -313,6 +313,12 @@ def test_launch_plan_of_the_named_shapes(monkeypatch):
     assert (wan.rows_per_workgroup, wan.whole_tiles, wan.ranges, wan.claimers, wan.counter) == (384, 768, 256, 256, 0)
     ring_chunk = _plan(1, 24, 4608, 1152)
     assert (ring_chunk.rows_per_workgroup, ring_chunk.ranges, ring_chunk.workgroups) == (256, 0, 432)
+    # tensors of a smaller head_dim run on the kernel built for the next one up, same geometry
+    fields = [n for n, _ in _lib.LaunchPlan._fields_]
+    for small, built in ((72, 128), (120, 128), (8, 64), (40, 64)):
+        for shape in ((2, 16, 4096, 4096), (1, 5, 20000, 20000, 77)):
+            a_, b_ = _plan(*shape, D=small), _plan(*shape, D=built)
+            assert [getattr(a_, n) for n in fields] == [getattr(b_, n) for n in fields], (small, shape)
     p = _lib.LaunchPlan()
     p.struct_size = 4
     a = _attn_args()

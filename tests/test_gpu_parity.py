@@ -61,7 +61,8 @@ def test_attn_16bit_small_vs_oracle(gpu, dtype, layout, B, H, Sq, Sk, D):
                                       (torch.bfloat16, 72), (torch.float16, 40), (torch.bfloat16, 96)])
 @pytest.mark.parametrize("Sq,Sk", [(1, 1), (33, 31), (130, 200), (128, 32)])
 def test_attn_generic_path_vs_oracle(gpu, dtype, D, Sq, Sk):
-    """fp32 inputs and head dims outside {64,128} run on the fp32 matrix cores."""
+    """fp32 inputs run on the fp32 matrix cores at any head_dim; the 16-bit cases here take the
+    16-bit kernel built for the next head_dim up (64 or 128)."""
     g = torch.Generator().manual_seed(D * 100 + Sq)
     q = torch.randn(2, 2, Sq, D, generator=g).to(dtype)
     k = torch.randn(2, 2, Sk, D, generator=g).to(dtype)
@@ -172,7 +173,7 @@ def test_claimed_ranges_vs_plain_launch_and_fp32(gpu, force_rows, kind, rows, Sk
 
 
 @pytest.mark.parametrize("rows", [128, 256, 384])
-@pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8", "bf16-d64", "fp16-d64"])
+@pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8", "bf16-d64", "fp16-d64", "bf16-d72", "fp16-d40", "fp16-d96", "bf16-d120", "bf16-d8"])
 @pytest.mark.parametrize("B,H,Sq,Sk,Sk2", [
     (1, 2, 1000, 777, 0),       # several workgroups per head, partial last query tile and KV tile
     (1, 1, 385, 8192, 0),       # balanced launch: KV ranges shared between workgroups
@@ -180,10 +181,11 @@ def test_claimed_ranges_vs_plain_launch_and_fp32(gpu, force_rows, kind, rows, Sk
     (2, 2, 50, 64, 1),          # fewer query rows than one workgroup covers
 ])
 def test_workgroup_shapes_vs_oracle(gpu, force_rows, rows, kind, B, H, Sq, Sk, Sk2):
-    """Every workgroup shape of the 16-bit (head_dim 128 and 64) and fp8 kernels, with and without
-    the balanced launch, against the oracle on the same inputs."""
+    """Every workgroup shape of the 16-bit (built for head_dim 128 and 64, also on tensors of a
+    smaller head_dim) and fp8 kernels, with and without the balanced launch, against the oracle on
+    the same inputs."""
     force_rows(rows)
-    D = 64 if kind.endswith("-d64") else 128
+    D = int(kind.split("-d")[1]) if "-d" in kind else 128
     kind = kind.split("-")[0]
     g = torch.Generator().manual_seed(rows + Sq + Sk)
     mk = lambda n: torch.randn(B, H, n, D, generator=g)
@@ -397,10 +399,42 @@ def test_update_out_and_lse_matches_oracle_layout(gpu):
     assert out.shape == (B, S, H, D) and lse.shape == (B, S, H, 1) and out.dtype == torch.float32
     assert _err(out, rout) <= 5e-6 and _err(lse, rlse) <= 5e-6
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [128, 256, 384])
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 72), (torch.float16, 88), (torch.bfloat16, 40), (torch.float16, 16)])
+def test_smaller_head_dim_touches_only_its_columns(gpu, force_rows, rows, dtype, D):
+    """Tensors of a head_dim below the one the 16-bit kernel is built for: the kernel must neither
+    read nor write the columns they do not have.  q, k, v and out are views of wider tensors whose
+    other columns hold NaN (a read would poison the result, a write would clear the NaN)."""
+    force_rows(rows)
+    W = 136
+    B, H, Sq = 1, 2, 500
+    g = torch.Generator().manual_seed(rows + D)
+    for Sk, balance in ((333, True), (8192, True), (8192, False)):
+        wide = lambda n: torch.full((B, H, n, W), float("nan"), dtype=dtype, device=gpu)
+        qw, kw_, vw, ow = wide(Sq), wide(Sk), wide(Sk), wide(Sq)
+        q, k, v = (torch.randn(B, H, n, D, generator=g).to(dtype) for n in (Sq, Sk, Sk))
+        qw[..., 8:8 + D], kw_[..., 16:16 + D], vw[..., :D] = q.to(gpu), k.to(gpu), v.to(gpu)
+        out = ow[..., 24:24 + D]
+        o, l = ops.attn_fwd(qw[..., 8:8 + D], kw_[..., 16:16 + D], vw[..., :D], out=out, balance=balance)
+        ro, rl = O.attn_fwd_ref(q, k, v)
+        assert _err(out, ro) <= TOL[dtype][0] and _err(l, rl) <= TOL[dtype][1]
+        assert torch.isnan(ow[..., :24]).all() and torch.isnan(ow[..., 24 + D:]).all()
+        # the same through the fused ring step: accumulator and final output inside NaN frames
+        aw = torch.full((B, H, Sq, W), float("nan"), device=gpu)
+        acc_o, acc_l = aw[..., 4:4 + D], torch.empty(B, H, Sq, device=gpu)
+        fw = wide(Sq)
+        ops.attn_fwd_accumulate(qw[..., 8:8 + D], kw_[..., 16:16 + D], vw[..., :D], acc_o, acc_l, first=True, final_out=fw[..., 8:8 + D])
+        po, pl = (out, l) if not balance else ops.attn_fwd(qw[..., 8:8 + D], kw_[..., 16:16 + D], vw[..., :D], balance=False)
+        assert torch.equal(fw[..., 8:8 + D], po) and torch.equal(acc_l, pl) and torch.equal(acc_o, po.float())
+        assert torch.isnan(aw[..., :4]).all() and torch.isnan(aw[..., 4 + D:]).all()
+        assert torch.isnan(fw[..., :8]).all() and torch.isnan(fw[..., 8 + D:]).all()
+
 
 # ---------------------------------------------------------------------------- fused ring step
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64)])
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64),
+                                      (torch.bfloat16, 72), (torch.float16, 104), (torch.float16, 24)])
 @pytest.mark.parametrize("layout", ["bhsd", "bshd"])
 def test_fused_ring_step_equals_forward_plus_merge(gpu, force_rows, dtype, D, layout):
     """xdit_attn_fwd_accumulate = xdit_attn_fwd + xdit_lse_merge, bit for bit, over three steps
@@ -410,7 +444,7 @@ def test_fused_ring_step_equals_forward_plus_merge(gpu, force_rows, dtype, D, la
     g = torch.Generator().manual_seed(D + Sq)
     q = torch.randn(B, H, Sq, D, generator=g).to(dtype)
     chunks = [(torch.randn(B, H, n, D, generator=g).to(dtype), torch.randn(B, H, n, D, generator=g).to(dtype)) for n in (257, 64, 130)]
-    for rows in ((128, 256, 384) if D == 128 else (128,)):
+    for rows in (128, 256, 384):
         force_rows(rows)
         qd = _layout(q, layout, gpu)
         acc_o = _layout(torch.full((B, H, Sq, D), float("nan")), layout, gpu)

@@ -52,15 +52,24 @@ int check_tensor(const char* name, const void* p, const xdit_strides& st, int es
   return 0;
 }
 
-// Query rows per workgroup (head_dim 128 and 64: 384, 256 or 128, i.e. 12, 8 or 4 wavefronts
-// sharing each K/V tile; other head_dims: 128).  Picks the shape with the shortest estimated critical path: KV iterations of the
+// Query rows per workgroup of the 16-bit and fp8 kernels: 384, 256 or 128, i.e. 12, 8 or 4
+// wavefronts sharing each K/V tile.  Picks the shape with the shortest estimated critical path: KV iterations of the
 // busiest compute unit (whole rounds of resident workgroups, or the balanced launch's shared last
 // round plus its fixed cost) times the rows a compute unit works on per iteration, with a small
 // penalty for the shapes that share a tile between fewer wavefronts.  Measured on Flux-1024
 // (72 KV tiles: 384 rows wins through the balanced launch) and on its ring chunks (18 KV tiles:
 // 256 rows, 0.079 ms against 0.101 ms at 384).
+// head_dim the 16-bit MFMA kernel is built for that holds a tensor head_dim of D (64 or 128; the
+// kernel treats the columns the tensors do not have as zeros), 0 if there is none.
+int kernel_head_dim(int D) { return D <= 0 || D % 8 != 0 || D > 128 ? 0 : (D <= 64 ? 64 : 128); }
+
+bool mfma16_path(const xdit_attn_args* a) {
+  return (a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && kernel_head_dim(a->D) != 0;
+}
+
 int rows_per_block_16(const xdit_attn_args* a) {
-  if (a->D != 128 && a->D != 64) return 128;
+  const int D = kernel_head_dim(a->D);
+  if (D == 0) return 128;
   const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128", "256" or "384": testing aid, read per call
   if (force != nullptr) {
     const int r = std::atoi(force);
@@ -76,7 +85,7 @@ int rows_per_block_16(const xdit_attn_args* a) {
   // 103 / 96 / 79 us), so the number of rounds decides
   static const double kPenalty128[3] = {1.0, 1.06, 1.12};
   static const double kPenalty64[3] = {1.0, 1.10, 1.0};
-  const double* kPenalty = a->D == 64 ? kPenalty64 : kPenalty128;
+  const double* kPenalty = D == 64 ? kPenalty64 : kPenalty128;
   int best = 128;
   double best_cost = 0;
   for (int i = 0; i < 3; i++) {
@@ -88,10 +97,10 @@ int rows_per_block_16(const xdit_attn_args* a) {
     xdit::AttnParams q;
     std::memset(&q, 0, sizeof(q));
     q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
-    xdit::plan_split(q, rows, slots, a->D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup);
+    xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup);
     // every segment costs a few iterations' worth of prologue and epilogue (about 13 us: 5
     // iterations at head_dim 128, 9 at head_dim 64), the combine pass about as much again
-    const double ovh = a->D == 64 ? 9.0 : 5.0;
+    const double ovh = D == 64 ? 9.0 : 5.0;
     const double units = q.split_units ? (double)(q.split_full / slots) * (nt + ovh) + q.split_share + 2 * ovh
                                        : (double)((tiles + slots - 1) / slots) * (nt + ovh);
     int64_t sharing = (tiles + cus - 1) / cus;  // workgroups on the busiest compute unit at once
@@ -202,8 +211,8 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   if (acc != nullptr) {
     if (acc->struct_size != sizeof(xdit_ring_acc))
       return fail(XDIT_ERR_INVALID_ARG, "acc struct_size %u != %zu (ABI mismatch)", acc->struct_size, sizeof(xdit_ring_acc));
-    if (!((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64)))
-      return fail(XDIT_ERR_UNSUPPORTED, "the fused ring step needs bf16 or fp16 inputs with head_dim 64 or 128");
+    if (!mfma16_path(a))
+      return fail(XDIT_ERR_UNSUPPORTED, "the fused ring step needs bf16 or fp16 inputs with head_dim at most 128");
     if ((rc = check_tensor("acc_out", acc->acc_out, acc->acc_out_stride, 4, a->D))) return rc;
     if (acc->acc_lse == nullptr) return fail(XDIT_ERR_INVALID_ARG, "acc_lse is NULL");
     if (acc->acc_lse_stride.b < 0 || acc->acc_lse_stride.h < 0 || acc->acc_lse_stride.s <= 0)
@@ -242,8 +251,9 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   hipStream_t stream = (hipStream_t)a->stream;
 
   hipError_t e;
-  if ((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64)) {
-    e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, a->D, rows_per_block_16(a), stream);
+  if (mfma16_path(a)) {
+    p.d_actual = a->D;
+    e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a), stream);
   } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
     if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
     e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, rows_per_block_16(a), stream);
@@ -277,8 +287,8 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   if (a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128) return (int64_t)xdit::attn_fwd_fp8_workspace(p, rows_per_block_16(a));
-  if (!((a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64))) return 0;
-  return (int64_t)xdit::attn_fwd_16_workspace(p, a->D, rows_per_block_16(a));
+  if (!mfma16_path(a)) return 0;
+  return (int64_t)xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows_per_block_16(a));
 }
 
 int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
@@ -292,13 +302,13 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
       a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30))
     return fail(XDIT_ERR_INVALID_ARG, "bad shape");
   const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128;
-  const bool b16 = (a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && (a->D == 128 || a->D == 64);
+  const bool b16 = mfma16_path(a);
   if (!fp8 && !b16) return fail(XDIT_ERR_UNSUPPORTED, "no launch plan for this dtype / head_dim (generic kernel: one workgroup per 64 query rows)");
   xdit::AttnParams p, q;
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   const int rows = rows_per_block_16(a);
-  const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q) : xdit::attn_fwd_16_workspace(p, a->D, rows, &q);
+  const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q);
   const uint32_t size = out->struct_size;
   std::memset(out, 0, sizeof(*out));
   out->struct_size = size;

@@ -1,4 +1,5 @@
-// Non-causal attention forward for 16-bit inputs (bf16 / fp16) on gfx950, head_dim 64 or 128.
+// Non-causal attention forward for 16-bit inputs (bf16 / fp16) on gfx950, built for head_dim 64 and 128
+// (tensors of a smaller head_dim, a multiple of 8, run on the next one up: see PAD below).
 //
 // Work decomposition
 //   workgroup = 256 threads = 4 wavefronts; it owns 128 query rows of one (batch, head);
@@ -37,7 +38,10 @@ constexpr int kPrefetch = 4;
 // whose KV range is shared between workgroups, and its normalised partial output (in T) and
 // log-sum-exp go to the workspace slot (part_out, part_lse), [row][D] and [row], to be folded by
 // attn_combine_kernel.
-template <typename T, int D, int NW>
+// PAD: the tensors' head_dim (p.d_actual, a multiple of 8) is smaller than D; the missing columns
+// are zeros in the Q fragments and in LDS (cleared here, never written by the tile loads) and are
+// not stored.
+template <typename T, int D, int NW, bool PAD>
 __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char* smem, const int tile,
                                              const int it0, const int it1, T* part_out, float* part_lse) {
   constexpr int kWaves = NW;
@@ -63,9 +67,17 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   const int qrow = qt * kRowsPerBlock + wave * kRowsPerWave + l32;
   const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
   const T* qptr = (const T*)p.q + b * p.qs_b + h * p.qs_h + (int64_t)qrow_c * p.qs_s + hh * 8;
+  const int dact = PAD ? p.d_actual : D;
   vec8 qf[KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ks++) qf[ks] = *(const vec8*)(qptr + ks * 16);
+  for (int ks = 0; ks < KSTEPS; ks++) {
+    if (!PAD || ks * 16 + hh * 8 < dact) {
+      qf[ks] = *(const vec8*)(qptr + ks * 16);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) qf[ks][e] = (T)0.f;
+    }
+  }
 
   // ---- direct global->LDS tile loads ------------------------------------------------------
   // A tile is 2*NG pieces of 1 KiB (K pieces 0..NG-1, then V pieces): piece g of K (or V) holds
@@ -84,6 +96,7 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   static_assert(G::NG % LW == 0, "pieces must divide evenly over the loader wavefronts");
   const int ld_row0 = G::NG * (lane / LANES_PER_ROW) + wave;  // row of this lane in pair 0
   const unsigned ld_colb = (lane % LANES_PER_ROW) * 16;       // byte offset inside the row
+  const bool ld_on = !PAD || ld_colb < (unsigned)dact * 2;    // lanes of columns the tensors do not have stay idle
   const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS unsigned char*)smem;
   const unsigned ld_kdst = lds_base + wave * G::K_PITCH;      // LDS address of K piece `wave`, buffer 0
   const unsigned ld_vdst = lds_base + G::K_BYTES + wave * G::V_PITCH;
@@ -115,7 +128,7 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   };
   // Loads the tile at the stream position into buffer `buf` and advances the position.
   auto issue_tile = [&](int t, int buf) {
-    if (kWaves == LW || wave < LW) {
+    if ((kWaves == LW || wave < LW) && ld_on) {
       const int last = (ld_left < kKeysPerTile ? ld_left : kKeysPerTile) - 1;
       const unsigned bo = buf * G::BUF_BYTES;
 #pragma unroll
@@ -159,6 +172,12 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
 
+  if (PAD) {  // zero the columns that no load writes (all of both buffers: simplest)
+    typedef __attribute__((ext_vector_type(4))) int i32x4;
+    const i32x4 zero = {0, 0, 0, 0};
+    for (int i = tid * 16; i < 2 * G::BUF_BYTES; i += 64 * kWaves * 16) *(XDIT_LDS i32x4*)((XDIT_LDS unsigned char*)smem + i) = zero;
+    __syncthreads();
+  }
   seek_tile(it0);
   issue_tile(it0, 0);
   // Make the compiler account for the Q fragment loads here, before the loop: the tile loads
@@ -299,7 +318,7 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
         f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
                    oacc[db][4 * a + 3] * inv};
         vec4 ov = __builtin_convertvector(o, vec4);
-        *(vec4*)(optr + 32 * db + 8 * a + 4 * hh) = ov;
+        if (!PAD || part_out != nullptr || 32 * db + 8 * a + 4 * hh < dact) *(vec4*)(optr + 32 * db + 8 * a + 4 * hh) = ov;
       }
     if (hh == 0) {
       if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
@@ -324,6 +343,7 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
       for (int a = 0; a < 4; a++) {
         typedef __attribute__((ext_vector_type(4))) T vec4;
         const int d = 32 * db + 8 * a + 4 * hh;
+        if (PAD && d >= dact) continue;
         f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
                    oacc[db][4 * a + 3] * inv};
         f32x4 m = __builtin_convertvector(__builtin_convertvector(o, vec4), f32x4);
@@ -342,11 +362,11 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   }
 }
 
-template <typename T, int D, int NW>
+template <typename T, int D, int NW, bool PAD>
 __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(const AttnParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // 2 x [K tile | V tile]
   run_workgroup<T, kRowsPerWave * NW, D>(p, [&](int tile, int it0, int it1, T* part_out, float* part_lse) {
-    attn_segment<T, D, NW>(p, smem, tile, it0, it1, part_out, part_lse);
+    attn_segment<T, D, NW, PAD>(p, smem, tile, it0, it1, part_out, part_lse);
   });
 }
 
@@ -354,8 +374,21 @@ __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(
 // workgroups per CU, one otherwise.
 static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 2 : 1); }
 
+template <typename T, int D, int NW, bool PAD>
+static hipError_t launch_kernel(const AttnParams& q, hipStream_t stream) {
+  static bool lds_ready = false;
+  constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
+  if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, NW, PAD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    lds_ready = true;
+  }
+  hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, NW, PAD>), dim3(split_grid(q)), dim3(64 * NW), lds, stream, q);
+  return hipSuccess;
+}
+
 template <typename T, int D, int NW>
-static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_ready) {
+static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   AttnParams q = p;
   constexpr int rows = 32 * NW;
   q.nq_tiles = (p.Sq + rows - 1) / rows;
@@ -363,14 +396,9 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream, bool& lds_
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
   bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup), rows, D, 2);
   if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
-  dim3 grid(split_grid(q));
-  constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
-  if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return e;
-    lds_ready = true;
-  }
-  hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, NW>), grid, dim3(64 * NW), lds, stream, q);
+  if (q.d_actual == D) q.d_actual = 0;
+  const hipError_t e = q.d_actual != 0 ? launch_kernel<T, D, NW, true>(q, stream) : launch_kernel<T, D, NW, false>(q, stream);
+  if (e != hipSuccess) return e;
   if (q.split_units) {
     const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
     const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
@@ -404,23 +432,21 @@ size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block, Att
 }
 
 // Host-side launcher (called from the C ABI after argument validation).
-// rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12 wavefronts), for head_dim 128 and 64.
-hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream) {
-  static bool ready[12] = {false, false, false, false, false, false, false, false, false, false, false, false};
-  if (D == 128 && rows_per_block == 384) {
-    return dtype_is_fp16 ? launch_one<_Float16, 128, 12>(p, stream, ready[6]) : launch_one<__bf16, 128, 12>(p, stream, ready[7]);
-  } else if (D == 128 && rows_per_block == 256) {
-    return dtype_is_fp16 ? launch_one<_Float16, 128, 8>(p, stream, ready[4]) : launch_one<__bf16, 128, 8>(p, stream, ready[5]);
-  } else if (D == 128) {
-    return dtype_is_fp16 ? launch_one<_Float16, 128, 4>(p, stream, ready[0]) : launch_one<__bf16, 128, 4>(p, stream, ready[1]);
-  } else if (D == 64 && rows_per_block == 384) {
-    return dtype_is_fp16 ? launch_one<_Float16, 64, 12>(p, stream, ready[10]) : launch_one<__bf16, 64, 12>(p, stream, ready[11]);
-  } else if (D == 64 && rows_per_block == 256) {
-    return dtype_is_fp16 ? launch_one<_Float16, 64, 8>(p, stream, ready[8]) : launch_one<__bf16, 64, 8>(p, stream, ready[9]);
-  } else if (D == 64) {
-    return dtype_is_fp16 ? launch_one<_Float16, 64, 4>(p, stream, ready[2]) : launch_one<__bf16, 64, 4>(p, stream, ready[3]);
-  }
+// D: the head_dim the kernel is built for, 128 or 64; p.d_actual, if not 0, is the tensors'
+// smaller head_dim (a multiple of 8).  rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12).
+template <typename T>
+static hipError_t launch_typed(const AttnParams& p, int D, int rows_per_block, hipStream_t stream) {
+  if (D == 128 && rows_per_block == 384) return launch_one<T, 128, 12>(p, stream);
+  if (D == 128 && rows_per_block == 256) return launch_one<T, 128, 8>(p, stream);
+  if (D == 128) return launch_one<T, 128, 4>(p, stream);
+  if (D == 64 && rows_per_block == 384) return launch_one<T, 64, 12>(p, stream);
+  if (D == 64 && rows_per_block == 256) return launch_one<T, 64, 8>(p, stream);
+  if (D == 64) return launch_one<T, 64, 4>(p, stream);
   return hipErrorInvalidValue;
+}
+
+hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream) {
+  return dtype_is_fp16 ? launch_typed<_Float16>(p, D, rows_per_block, stream) : launch_typed<__bf16>(p, D, rows_per_block, stream);
 }
 
 }  // namespace xdit

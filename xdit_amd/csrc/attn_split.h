@@ -97,6 +97,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, c
   const int row = local / TPR;
   const int col = (local - row * TPR) * 8;
   if (row >= rows_per_block) return;
+  if (p.d_actual != 0 && col >= p.d_actual) return;  // columns the tensors do not have
   const int tile = p.split_full + r;
   const int bh = tile / p.nq_tiles;
   const int qt = tile - bh * p.nq_tiles;

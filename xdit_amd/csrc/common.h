@@ -50,6 +50,7 @@ struct AttnParams {
   int total_tiles;    // B * H * nq_tiles
   int tiles_per_xcd;  // ceil(total_tiles / 8)
   float scale;        // softmax scale
+  int d_actual;       // head_dim of the tensors when the kernel is built for a larger one (0: the kernel's own)
   // balanced launch (see attn_fwd_16_kernel); all zero for a plain launch
   int split_full;     // query tiles handled whole, by the first workgroups
   int split_units;    // workgroups sharing the KV iterations of the remaining query tiles

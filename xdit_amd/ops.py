@@ -163,8 +163,8 @@ def launch_plan(q, k, k2=None):
 
 
 def fused_ring_step_supported(q):
-    """Whether `attn_fwd_accumulate` takes these queries (bf16 / fp16, head_dim 64 or 128)."""
-    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] in (64, 128)
+    """Whether `attn_fwd_accumulate` takes these queries (bf16 / fp16, head_dim a multiple of 8 up to 128)."""
+    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] % 8 == 0 and 0 < q.shape[-1] <= 128
 
 
 def attn_fwd_accumulate(q, k, v, acc_out, acc_lse, first=False, final_out=None, discard_acc_out=False,
