@@ -40,8 +40,10 @@ constexpr int kPrefetch = 4;
 // attn_combine_kernel.
 // PAD: the tensors' head_dim (p.d_actual, a multiple of 8) is smaller than D; the missing columns
 // are zeros in the Q fragments and in LDS (cleared here, never written by the tile loads) and are
-// not stored.
-template <typename T, int D, int NW, bool PAD>
+// not stored.  DC (a multiple of 32, d_actual <= DC <= D) is the head_dim the two products are
+// computed over: LDS tiles keep the geometry of D, contraction steps and output blocks past DC
+// are left out.
+template <typename T, int D, int DC, int NW, bool PAD>
 __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char* smem, const int tile,
                                              const int it0, const int it1, T* part_out, float* part_lse) {
   constexpr int kWaves = NW;
@@ -49,8 +51,9 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   typedef typename Mfma16<T>::vec8 vec8;
   typedef typename Mfma16<T>::vec2 vec2;
   typedef TileGeom<D> G;
-  constexpr int KSTEPS = D / 16;         // contraction steps of QK^T
-  constexpr int DBLOCKS = D / 32;        // 32-row blocks of O^T
+  static_assert(DC % 32 == 0 && DC <= D && (PAD || DC == D), "computed head_dim");
+  constexpr int KSTEPS = DC / 16;        // contraction steps of QK^T
+  constexpr int DBLOCKS = DC / 32;       // 32-row blocks of O^T
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -362,11 +365,11 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   }
 }
 
-template <typename T, int D, int NW, bool PAD>
+template <typename T, int D, int DC, int NW, bool PAD>
 __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(const AttnParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // 2 x [K tile | V tile]
   run_workgroup<T, kRowsPerWave * NW, D>(p, [&](int tile, int it0, int it1, T* part_out, float* part_lse) {
-    attn_segment<T, D, NW, PAD>(p, smem, tile, it0, it1, part_out, part_lse);
+    attn_segment<T, D, DC, NW, PAD>(p, smem, tile, it0, it1, part_out, part_lse);
   });
 }
 
@@ -374,16 +377,16 @@ __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(
 // workgroups per CU, one otherwise.
 static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 2 : 1); }
 
-template <typename T, int D, int NW, bool PAD>
+template <typename T, int D, int DC, int NW, bool PAD>
 static hipError_t launch_kernel(const AttnParams& q, hipStream_t stream) {
   static bool lds_ready = false;
   constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
   if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, NW, PAD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, DC, NW, PAD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     lds_ready = true;
   }
-  hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, NW, PAD>), dim3(split_grid(q)), dim3(64 * NW), lds, stream, q);
+  hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, DC, NW, PAD>), dim3(split_grid(q)), dim3(64 * NW), lds, stream, q);
   return hipSuccess;
 }
 
@@ -397,7 +400,10 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup), rows, D, 2);
   if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
   if (q.d_actual == D) q.d_actual = 0;
-  const hipError_t e = q.d_actual != 0 ? launch_kernel<T, D, NW, true>(q, stream) : launch_kernel<T, D, NW, false>(q, stream);
+  constexpr int DS = D == 128 ? 96 : 32;  // the smaller computed head_dim built for this D
+  const hipError_t e = q.d_actual == 0    ? launch_kernel<T, D, D, NW, false>(q, stream)
+                       : q.d_actual <= DS ? launch_kernel<T, D, DS, NW, true>(q, stream)
+                                          : launch_kernel<T, D, D, NW, true>(q, stream);
   if (e != hipSuccess) return e;
   if (q.split_units) {
     const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
