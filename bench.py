@@ -2,6 +2,7 @@
 """Benchmark of the attention hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
+    python bench.py --model-shapes     (a table instead: see below)
 
 A "step" is one call of the joint-attention forward on the Flux-1024 shape
 (B=1, H=24, S=4608 = 512 text + 4096 image tokens, D=128, bf16, non-causal, BHSD-contiguous,
@@ -15,6 +16,11 @@ q/k per-head RMSNorm'd), inputs resident in HBM.  Prints ONE JSON line:
   also         the other named shapes: HunyuanVideo-720p head shard (bf16), Wan2.1 720p head
                shard (fp8), the 4-chunk ring with its fp32 merges, the merge kernel's GB/s, the
                fp8 quantiser and the fused norm + rotary prologue (GB/s against the HBM peak)
+               and torch's own GPU flash attention (the op behind the reference's default
+               SDPA_FLASH backend, attention_backend.py:504-516) on the same tensors and GPU
+--model-shapes prints, instead of the JSON line, one row per attention shape of the reference's
+model families (self, joint and cross attention; head_dim 128, 64, 72, 88): this library against
+torch's GPU flash attention on the same tensors, with the largest difference between the outputs.
 Everything runs on one GPU; --gpus above 1 is refused (this build has no multi-GPU path).
 """
 import argparse
@@ -71,6 +77,51 @@ def attn_flops(B, H, Sq, Sk, D):
     return 4.0 * B * H * Sq * Sk * D
 
 
+def torch_flash(q, k, v):
+    """torch's GPU flash attention: the call inside the reference's SDPA_FLASH adapter
+    (xfuser/core/distributed/attention_backend.py:504-516), its default backend."""
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+    with sdpa_kernel([SDPBackend.FLASH_ATTENTION]):
+        return torch.nn.functional.scaled_dot_product_attention(q, k, v, dropout_p=0.0, is_causal=False)
+
+
+# Attention calls of the reference's model families at their usual resolutions, bf16:
+# (name, B, H, Sq, Sk, D)
+MODEL_SHAPES = [
+    ("Flux-1024 joint", 1, 24, 4608, 4608, 128),
+    ("Flux-2048 joint", 1, 24, 16896, 16896, 128),
+    ("HunyuanVideo-720p, 3 of 24 heads", 1, 3, 119056, 119056, 128),
+    ("Wan2.1-480p self", 1, 40, 32760, 32760, 128),
+    ("Wan2.1-480p cross (512 text keys)", 1, 40, 32760, 512, 128),
+    ("SD3-1024 joint", 2, 24, 4250, 4250, 64),
+    ("CogVideoX-5B", 2, 48, 17776, 17776, 64),
+    ("PixArt-1024 self", 2, 16, 4096, 4096, 72),
+    ("PixArt-1024 cross (120 text keys)", 2, 16, 4096, 120, 72),
+    ("HunyuanDiT-1024 self", 2, 16, 4096, 4096, 88),
+]
+
+
+def model_shapes(dev):
+    from xdit_amd import ops
+    print("| shape | B H Sq Sk D | this library us | TFLOP/s | torch flash us | TFLOP/s | speed-up | max abs diff of out |")
+    print("|---|---|---|---|---|---|---|---|")
+    for name, B, H, Sq, Sk, D in MODEL_SHAPES:
+        g = torch.Generator(device="cpu").manual_seed(Sq + D)
+        q, k, v = (torch.randn(B, H, n, D, generator=g).bfloat16().to(dev) for n in (Sq, Sk, Sk))
+        fl = attn_flops(B, H, Sq, Sk, D)
+        steps, warm = (5, 3) if fl > 5e12 else (20, 40)
+        _, ms = time_calls(lambda: ops.attn_fwd(q, k, v), steps, warm)
+        o, _ = ops.attn_fwd(q, k, v)
+        try:
+            ro = torch_flash(q, k, v)
+            _, rms = time_calls(lambda: torch_flash(q, k, v), steps, min(warm, 10))
+            ref = "%.1f | %.0f | %.2fx | %.4f" % (rms * 1e3, fl / rms / 1e9, rms / ms, (ro.float() - o.float()).abs().max().item())
+        except Exception as e:  # the comparison is optional: report, do not fail
+            ref = "failed: %s | | |" % str(e)[:60]
+        print("| %s | %d %d %d %d %d | %.1f | %.0f | %s |" % (name, B, H, Sq, Sk, D, ms * 1e3, fl / ms / 1e9, ref), flush=True)
+        del q, k, v, o
+
+
 def cpu_baseline(q, k, v, budget_s=12.0):
     """The reference's CPU SDPA path on the same Flux-1024 tensors (all heads, fp32), repeated
     for about `budget_s` seconds of CPU work; reports the median run."""
@@ -106,6 +157,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--model-shapes", action="store_true",
+                    help="print a table of the reference's model shapes against torch's GPU flash attention, and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof byte counters)")
     args = ap.parse_args()
@@ -121,6 +174,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.model_shapes:
+        model_shapes(dev)
+        return
     B, H, S, D = 1, 24, 4608, 128
     q, k, v = make_inputs(B, H, S, D, 1002, dev)
     out = torch.empty_like(q)
@@ -177,6 +233,12 @@ def main():
         ob = torch.empty(q.shape[0], q.shape[2], q.shape[1], q.shape[3], dtype=q.dtype, device=q.device).transpose(1, 2)
         _, ms = time_calls(lambda: ops.attn_fwd(qb, kb, vb, out=ob), args.steps, args.warmup)
         also["c2_flux1024_bshd_view"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        # torch's GPU flash attention on the same tensors: what the reference's default backend runs
+        try:
+            _, ms = time_calls(lambda: torch_flash(q, k, v), args.steps, args.warmup)
+            also["c2_flux1024_torch_flash_same_gpu"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        except Exception as e:
+            also["c2_flux1024_torch_flash_same_gpu"] = {"error": str(e)[:120]}
         # ring of 4 KV chunks, merged in fp32 (the cast of the last fold is fused)
         fn = usp._get_attention_function()
         _, ms = time_calls(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), n, 3)
@@ -217,6 +279,11 @@ def main():
         fl = attn_flops(Bh, Hh, Sh, Sh, D)
         also["c4_hunyuan720p_shard"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1),
                                         "frac_bf16_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        try:
+            _, ms = time_calls(lambda: torch_flash(qh, kh, vh), 5, 2)
+            also["c4_hunyuan720p_shard_torch_flash_same_gpu"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1)}
+        except Exception as e:
+            also["c4_hunyuan720p_shard_torch_flash_same_gpu"] = {"error": str(e)[:120]}
         del qh, kh, vh
         # Wan2.1 720p head shard, fp8 e4m3fn + per-head scales -> bf16
         Bw, Hw, Sw = 1, 5, 75600
