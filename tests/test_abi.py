@@ -319,6 +319,12 @@ def test_launch_plan_of_the_named_shapes(monkeypatch):
         for shape in ((2, 16, 4096, 4096), (1, 5, 20000, 20000, 77)):
             a_, b_ = _plan(*shape, D=small), _plan(*shape, D=built)
             assert [getattr(a_, n) for n in fields] == [getattr(b_, n) for n in fields], (small, shape)
+    # a problem too large for one launch is refused by the planning calls as by the launch
+    big = _attn_args(B=40000, H=40000, Sq=64)
+    p = _lib.LaunchPlan()
+    p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
+    assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(big), ctypes.byref(p)) == _lib.XDIT_ERR_INVALID_ARG
+    assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(big)) == _lib.XDIT_ERR_INVALID_ARG
     p = _lib.LaunchPlan()
     p.struct_size = 4
     a = _attn_args()

@@ -281,7 +281,8 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
   if (a->struct_size != sizeof(xdit_attn_args))
     return fail(XDIT_ERR_INVALID_ARG, "struct_size %u != %zu (ABI mismatch)", a->struct_size, sizeof(xdit_attn_args));
   if (a->B <= 0 || a->H <= 0 || a->Sq <= 0 || a->Sk <= 0 || a->Sk2 < 0 || a->Sq > (int64_t(1) << 30) ||
-      a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30))
+      a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30) ||
+      (int64_t)a->B * a->H * ((a->Sq + 31) / 32) > (int64_t(1) << 30))
     return fail(XDIT_ERR_INVALID_ARG, "bad shape");
   xdit::AttnParams p;
   std::memset(&p, 0, sizeof(p));
@@ -299,7 +300,8 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
   if (out->struct_size != sizeof(xdit_launch_plan))
     return fail(XDIT_ERR_INVALID_ARG, "plan struct_size %u != %zu (ABI mismatch)", out->struct_size, sizeof(xdit_launch_plan));
   if (a->B <= 0 || a->H <= 0 || a->Sq <= 0 || a->Sk <= 0 || a->Sk2 < 0 || a->Sq > (int64_t(1) << 30) ||
-      a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30))
+      a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30) ||
+      (int64_t)a->B * a->H * ((a->Sq + 31) / 32) > (int64_t(1) << 30))
     return fail(XDIT_ERR_INVALID_ARG, "bad shape");
   const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128;
   const bool b16 = mfma16_path(a);
