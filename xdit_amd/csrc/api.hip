@@ -259,7 +259,7 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
     e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, rows_per_block_16(a), stream);
   } else {
     if (a->D > 128) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d above 128 is not implemented", a->D);
-    e = xdit::launch_attn_fwd_f32(p, a->dtype, a->D, stream);
+    e = xdit::launch_attn_fwd_f32(p, a->D, stream);  // fp32 tensors: every 16-bit case went to the 16-bit kernel
   }
   if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
   return XDIT_OK;

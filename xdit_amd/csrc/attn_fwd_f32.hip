@@ -1,8 +1,7 @@
-// Generic non-causal attention forward computed on the fp32 matrix cores
-// (v_mfma_f32_32x32x2_f32) for gfx950: fp32 / bf16 / fp16 inputs, any head_dim that is a
-// multiple of 8 up to 128 (e.g. 72).  Inputs are converted to fp32 while they are staged into
-// LDS, so the products are exact fp32 products; this is the path for fp32 tensors and for head
-// dims the 16-bit kernel does not cover.  Same orientation as the 16-bit kernel:
+// Non-causal attention forward for fp32 tensors on the fp32 matrix cores
+// (v_mfma_f32_32x32x2_f32) of gfx950, any head_dim that is a multiple of 8 up to 128 (e.g. 72):
+// exact fp32 products, fp32 accumulation.  (16-bit tensors of every such head_dim run on the
+// 16-bit kernel.)  Same orientation as the 16-bit kernel:
 //   S^T = K Q^T  (A = K rows, B = Q^T in registers),  O^T = V^T P^T  (B = P^T = the S^T registers).
 // With a contraction depth of 2 per instruction every operand is ONE float per lane, so V^T is a
 // plain LDS read (lanes along head_dim) and needs no transposing load.
@@ -24,18 +23,13 @@ template <> __device__ __forceinline__ void load8<float>(const float* p, float (
   f32x4 a = ((const f32x4*)p)[0], b = ((const f32x4*)p)[1];
   for (int i = 0; i < 4; i++) { x[i] = a[i]; x[4 + i] = b[i]; }
 }
-template <> __device__ __forceinline__ void load8<__bf16>(const __bf16* p, float (&x)[8]) {
-  bf16x8 v = *(const bf16x8*)p;
-  for (int i = 0; i < 8; i++) x[i] = (float)v[i];
-}
-template <> __device__ __forceinline__ void load8<_Float16>(const _Float16* p, float (&x)[8]) {
-  f16x8 v = *(const f16x8*)p;
-  for (int i = 0; i < 8; i++) x[i] = (float)v[i];
-}
 
-// DB = number of 32-wide head_dim blocks (head_dim <= 32*DB; columns past head_dim are zero).
-template <typename T, int DB>
-__global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const AttnParams p, const int D) {
+// D8 = head_dim / 8.  The first product contracts exactly head_dim; the second works on 32-wide
+// blocks of head_dim (columns past head_dim are zero in LDS and are not stored).
+template <typename T, int D8>
+__global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const AttnParams p) {
+  constexpr int D = 8 * D8;
+  constexpr int DB = (D + 31) / 32;
   constexpr int DP = 32 * DB;       // padded head_dim
   constexpr int LD = DP + 1;        // LDS row stride in floats (odd: conflict-free column reads)
   constexpr int CHUNKS = DP / 8;    // 8-element chunks per padded row
@@ -145,7 +139,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const AttnParams p, c
 #pragma unroll
     for (int i = 0; i < 16; i++) sacc[i] = 0.f;
 #pragma unroll
-    for (int s = 0; s < DP / 2; s++) {
+    for (int s = 0; s < D / 2; s++) {
       const float kf = ks[l32 * LD + 2 * s + hh];
       sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf, qf[s], sacc, 0, 0, 0);
     }
@@ -204,32 +198,33 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const AttnParams p, c
   }
 }
 
+template <typename T, int D8>
+static void launch_d(const AttnParams& q, int d8, dim3 grid, hipStream_t stream) {
+  if constexpr (D8 <= 16) {
+    if (d8 == D8) hipLaunchKernelGGL((attn_fwd_f32_kernel<T, D8>), grid, dim3(256), 0, stream, q);
+    else launch_d<T, D8 + 1>(q, d8, grid, stream);
+  }
+}
+
 template <typename T>
 static hipError_t launch_t(const AttnParams& q, int D, dim3 grid, hipStream_t stream) {
-  const int db = (D + 31) / 32;
-  switch (db) {
-    case 1: hipLaunchKernelGGL((attn_fwd_f32_kernel<T, 1>), grid, dim3(256), 0, stream, q, D); break;
-    case 2: hipLaunchKernelGGL((attn_fwd_f32_kernel<T, 2>), grid, dim3(256), 0, stream, q, D); break;
-    case 3: hipLaunchKernelGGL((attn_fwd_f32_kernel<T, 3>), grid, dim3(256), 0, stream, q, D); break;
-    case 4: hipLaunchKernelGGL((attn_fwd_f32_kernel<T, 4>), grid, dim3(256), 0, stream, q, D); break;
-    default: return hipErrorInvalidValue;
-  }
+  if (D <= 0 || D % 8 != 0 || D > 128) return hipErrorInvalidValue;
+  launch_d<T, 1>(q, D / 8, grid, stream);
   return hipGetLastError();
 }
 
 }  // namespace f32path
 
-// dtype: 0 bf16, 1 fp16, 2 fp32.
-hipError_t launch_attn_fwd_f32(const AttnParams& p, int dtype, int D, hipStream_t stream) {
+// Workgroups of 128 query rows: smaller ones (64 or 32 rows, to fill the chip on small problems)
+// were measured and are not faster (PixArt-512 fp32, 16 x 1024 rows: 136 / 140 / 156 us): the
+// number of wavefronts, each bound by its own chain of MFMAs, stays the same.
+hipError_t launch_attn_fwd_f32(const AttnParams& p, int D, hipStream_t stream) {
   AttnParams q = p;
   q.nq_tiles = (p.Sq + f32path::kRowsPerBlock - 1) / f32path::kRowsPerBlock;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
   dim3 grid(q.tiles_per_xcd * 8);
-  if (dtype == 2) return f32path::launch_t<float>(q, D, grid, stream);
-  if (dtype == 0) return f32path::launch_t<__bf16>(q, D, grid, stream);
-  if (dtype == 1) return f32path::launch_t<_Float16>(q, D, grid, stream);
-  return hipErrorInvalidValue;
+  return f32path::launch_t<float>(q, D, grid, stream);
 }
 
 }  // namespace xdit

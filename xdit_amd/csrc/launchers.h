@@ -71,7 +71,7 @@ hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int
 size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block, AttnParams* plan = nullptr);
 hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream);
 size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan = nullptr);
-hipError_t launch_attn_fwd_f32(const AttnParams& p, int dtype, int D, hipStream_t stream);
+hipError_t launch_attn_fwd_f32(const AttnParams& p, int D, hipStream_t stream);  // fp32 tensors only
 hipError_t launch_fp8_quant(const QuantParams& p, int in_dtype, hipStream_t stream);
 hipError_t launch_qk_prologue(const PrologueParams& p, int dtype, hipStream_t stream);
 hipError_t launch_qk_prologue_batch(const PrologueBatch& b, int dtype, hipStream_t stream);
