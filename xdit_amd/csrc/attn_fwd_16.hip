@@ -40,9 +40,9 @@ constexpr int kPrefetch = 4;
 // attn_combine_kernel.
 // PAD: the tensors' head_dim (p.d_actual, a multiple of 8) is smaller than D; the missing columns
 // are zeros in the Q fragments and in LDS (cleared here, never written by the tile loads) and are
-// not stored.  DC (a multiple of 32, d_actual <= DC <= D) is the head_dim the two products are
-// computed over: LDS tiles keep the geometry of D, contraction steps and output blocks past DC
-// are left out.
+// not stored.  DC (a multiple of 16, d_actual <= DC <= D) is the head_dim the two products are
+// computed over: LDS tiles keep the geometry of D, contraction steps (of 16) and output blocks
+// (of 32) past DC are left out.
 template <typename T, int D, int DC, int NW, bool PAD>
 __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char* smem, const int tile,
                                              const int it0, const int it1, T* part_out, float* part_lse) {
@@ -51,9 +51,9 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   typedef typename Mfma16<T>::vec8 vec8;
   typedef typename Mfma16<T>::vec2 vec2;
   typedef TileGeom<D> G;
-  static_assert(DC % 32 == 0 && DC <= D && (PAD || DC == D), "computed head_dim");
-  constexpr int KSTEPS = DC / 16;        // contraction steps of QK^T
-  constexpr int DBLOCKS = DC / 32;       // 32-row blocks of O^T
+  static_assert(DC % 16 == 0 && DC <= D && (PAD || DC == D), "computed head_dim");
+  constexpr int KSTEPS = DC / 16;          // contraction steps of QK^T
+  constexpr int DBLOCKS = (DC + 31) / 32;  // 32-row blocks of O^T
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -400,10 +400,18 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup), rows, D, 2);
   if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
   if (q.d_actual == D) q.d_actual = 0;
-  constexpr int DS = D == 128 ? 96 : 32;  // the smaller computed head_dim built for this D
-  const hipError_t e = q.d_actual == 0    ? launch_kernel<T, D, D, NW, false>(q, stream)
-                       : q.d_actual <= DS ? launch_kernel<T, D, DS, NW, true>(q, stream)
-                                          : launch_kernel<T, D, D, NW, true>(q, stream);
+  // computed head_dims built for tensors smaller than D: 80, 96, 112 (and 128) of 128; 32 (and 64) of 64
+  hipError_t e;
+  if (q.d_actual == 0) {
+    e = launch_kernel<T, D, D, NW, false>(q, stream);
+  } else if constexpr (D == 128) {
+    e = q.d_actual <= 80    ? launch_kernel<T, D, 80, NW, true>(q, stream)
+        : q.d_actual <= 96  ? launch_kernel<T, D, 96, NW, true>(q, stream)
+        : q.d_actual <= 112 ? launch_kernel<T, D, 112, NW, true>(q, stream)
+                            : launch_kernel<T, D, 128, NW, true>(q, stream);
+  } else {
+    e = q.d_actual <= 32 ? launch_kernel<T, D, 32, NW, true>(q, stream) : launch_kernel<T, D, 64, NW, true>(q, stream);
+  }
   if (e != hipSuccess) return e;
   if (q.split_units) {
     const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
