@@ -216,7 +216,7 @@ def main():
             # HBM bytes per step from rocprofv3 FETCH_SIZE / WRITE_SIZE counters, each scaled by the
             # same counter's reading for a 256 MiB copy in the same run (--copy-calibration)
             "traffic": MEASURED_HBM_BYTES_PER_LAUNCH,
-            "kernel": "attn_fwd_16_kernel<bf16,128,12> (+ attn_combine_kernel<bf16,128> for the shared last round)",
+            "kernel": "attn_fwd_16_kernel<bf16,128,128,12,false> (+ attn_combine_kernel<bf16,128> for the shared last round)",
             "kernel_ms": round(ev_ms, 5),
         },
     }
