@@ -431,6 +431,56 @@ def test_smaller_head_dim_touches_only_its_columns(gpu, force_rows, rows, dtype,
         assert torch.isnan(fw[..., :8]).all() and torch.isnan(fw[..., 8 + D:]).all()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(8))
+def test_random_problems_vs_oracle(gpu, monkeypatch, seed):
+    """Random small problems over everything a call can vary: dtype, head_dim (every multiple of 8
+    up to 128), ragged lengths, a second KV segment, memory layout per tensor, softmax scale,
+    workgroup shape (forced or chosen by the library), balanced or plain launch, and the fused
+    ring step on top of an earlier block.  Every result is checked against the oracle."""
+    import random
+    rnd = random.Random(1000 + seed)
+    g = torch.Generator().manual_seed(seed)
+    for case in range(8):
+        dtype = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        D = 8 * rnd.randint(1, 16)
+        B, H = rnd.randint(1, 2), rnd.randint(1, 4)
+        Sq = rnd.choice([1, 7, 33, 128, 129, 300, 385, 700])
+        Sk = rnd.choice([1, 5, 64, 65, 200, 1000, 3000])
+        Sk2 = rnd.choice([0, 0, 1, 77, 256])
+        rows = rnd.choice([None, 128, 256, 384])
+        balance = rnd.random() < 0.7
+        scale = rnd.choice([None, 0.05, 0.2])
+        if rows is None:
+            monkeypatch.delenv("XDIT_ATTN_ROWS", raising=False)
+        else:
+            monkeypatch.setenv("XDIT_ATTN_ROWS", str(rows))
+        mk = lambda n: torch.randn(B, H, n, D, generator=g).to(dtype)
+        q, k, v = mk(Sq), mk(Sk), mk(Sk)
+        k2, v2 = (mk(Sk2), mk(Sk2)) if Sk2 else (None, None)
+        lay = lambda t: None if t is None else _layout(t, rnd.choice(["bhsd", "bshd"]), gpu)
+        what = (seed, case, dtype, D, B, H, Sq, Sk, Sk2, rows, balance, scale)
+        kall, vall = (k, v) if not Sk2 else (torch.cat([k, k2], 2), torch.cat([v, v2], 2))
+        ro, rl = O.attn_fwd_ref(q, kall, vall, scale)
+        qd, kd, vd, k2d, v2d = lay(q), lay(k), lay(v), lay(k2), lay(v2)
+        o, l = ops.attn_fwd(qd, kd, vd, softmax_scale=scale, k2=k2d, v2=v2d, balance=balance)
+        assert _err(o, ro) <= TOL[dtype][0] and _err(l, rl) <= TOL[dtype][1], what
+        if ops.fused_ring_step_supported(qd):
+            # an earlier block (the first Sk keys alone), then this call folded on top of it
+            bo, bl = ops.attn_fwd(qd, kd, vd, softmax_scale=scale)
+            acc_o, acc_l = torch.empty(B, H, Sq, D, device=gpu), torch.empty(B, H, Sq, device=gpu)
+            ops.lse_merge(acc_o, acc_l, bo, bl, first=True)
+            fin = torch.empty(B, H, Sq, D, dtype=dtype, device=gpu)
+            ops.attn_fwd_accumulate(qd, kd, vd, acc_o, acc_l, final_out=fin, softmax_scale=scale, k2=k2d, v2=v2d)
+            r1o, r1l = O.attn_fwd_ref(q, k, v, scale)
+            mo, ml = O.merge_ref(r1o.to(dtype).double(), r1l, ro.to(dtype), rl)
+            # two roundings to the 16-bit type (the block, then the result) on values that are not
+            # averages of many keys here and can reach 4-5 (half a unit in the last place of a bf16
+            # value in [4, 8) is 0.0156): 2^-7 relative to the largest value, where that is above 2e-2
+            tol = max(2e-2, 2.0 ** -7 * mo.abs().max().item())
+            assert _err(acc_o, mo) <= tol and _err(acc_l, ml) <= 1e-3 and _err(fin, mo) <= tol, what
+
+
 # ---------------------------------------------------------------------------- fused ring step
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64),
