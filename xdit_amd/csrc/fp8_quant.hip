@@ -79,8 +79,9 @@ __global__ void fill_zero_kernel(float* p, int n) {
 // division in the loop and the trip count is the same for every thread of a workgroup (the
 // lanes of a row exchange data in the Hadamard rotation).
 constexpr int kRowsInFlight = 4;
+constexpr int kAbsmaxRowsInFlight = 8;  // the read-only pass: nothing but loads to keep in flight
 
-template <typename T, typename F>
+template <typename T, int kRowsInFlight = quant::kRowsInFlight, typename F>
 __device__ __forceinline__ void for_each_chunk(const QuantParams& p, const T* x, F&& f) {
   const int cpr = p.D >> 3;
   const int rpb = 256 / cpr;              // rows per workgroup step
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(256) void absmax_kernel(const QuantParams p) {
   const int b = bh / p.H, h = bh - b * p.H;
   const T* x = (const T*)p.x + b * p.xs_b + h * p.xs_h;
   float m = 0.f;
-  for_each_chunk<T>(p, x, [&](float (&v)[8], int64_t, int, bool live) {
+  for_each_chunk<T, kAbsmaxRowsInFlight>(p, x, [&](float (&v)[8], int64_t, int, bool live) {
     if (live) {
 #pragma unroll
       for (int j = 0; j < 8; j++) m = fmaxf(m, fabsf(v[j]));  // fmaxf drops NaN operands
