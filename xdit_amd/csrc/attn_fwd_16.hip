@@ -379,12 +379,13 @@ static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 2 : 
 
 template <typename T, int D, int DC, int NW, bool PAD>
 static hipError_t launch_kernel(const AttnParams& q, hipStream_t stream) {
-  static bool lds_ready = false;
+  static std::atomic<bool> lds_ready[kMaxDevices];
   constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
-  if (!lds_ready) {  // > 64 KiB of dynamic LDS must be enabled once per kernel
+  const int slot = current_device_slot();
+  if (!lds_ready[slot].load(std::memory_order_relaxed)) {  // > 64 KiB of dynamic LDS must be enabled once per kernel and device
     hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, DC, NW, PAD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
-    lds_ready = true;
+    lds_ready[slot].store(true, std::memory_order_relaxed);
   }
   hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, DC, NW, PAD>), dim3(split_grid(q)), dim3(64 * NW), lds, stream, q);
   return hipSuccess;

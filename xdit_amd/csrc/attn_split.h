@@ -3,6 +3,8 @@
 // into equal ranges, one per workgroup; partial (out, lse) pairs go through a workspace and are
 // folded by attn_combine_kernel.
 #pragma once
+#include <atomic>
+
 #include "attn_tiles.h"
 
 namespace xdit {
@@ -150,15 +152,25 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, c
   if (col == 0 && p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = L + __logf(denom);
 }
 
-// Compute units of the current device (cached).
+// State cached per device (a process may drive several): index of the current device.
+constexpr int kMaxDevices = 64;
+static inline int current_device_slot() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) dev = 0;
+  return dev % kMaxDevices;
+}
+
+// Compute units of the current device (cached; concurrent first calls store the same value).
 static inline int resident_cus() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
+  static std::atomic<int> cus[kMaxDevices];
+  const int slot = current_device_slot();
+  int n = cus[slot].load(std::memory_order_relaxed);
+  if (n == 0) {
+    int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cus = n;
+    cus[slot].store(n, std::memory_order_relaxed);
   }
-  return cus;
+  return n;
 }
 
 // Ranges shorter than this many KV iterations are not worth a claim of their own (prologue,
