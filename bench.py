@@ -89,6 +89,7 @@ def torch_flash(q, k, v):
 # (name, B, H, Sq, Sk, D)
 MODEL_SHAPES = [
     ("Flux-1024 joint", 1, 24, 4608, 4608, 128),
+    ("Flux-1024 joint, 3 of 24 heads", 1, 3, 4608, 4608, 128),
     ("Flux-2048 joint", 1, 24, 16896, 16896, 128),
     ("HunyuanVideo-720p, 3 of 24 heads", 1, 3, 119056, 119056, 128),
     ("Wan2.1-480p self", 1, 40, 32760, 32760, 128),
