@@ -33,6 +33,11 @@ constexpr int kRowsPerWave = 32;
 // LDS fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
 constexpr int kPrefetch = 4;
 
+// Output staging block of a wavefront in the epilogue: 32 rows of 64 16-bit columns, rows 8 bytes
+// apart from a multiple of 128 so that the 8-byte writes of the 32 lanes of a half hit 32 banks.
+constexpr int kStagePitchBytes = 64 * 2 + 8;
+constexpr int kStageBytesPerWave = kRowsPerWave * kStagePitchBytes;
+
 // One segment of work: the query tile `tile`, KV tiles [it0, it1).  With `part_out == nullptr` the
 // normalised result goes to the output tensors; otherwise the segment is one PART of a query tile
 // whose KV range is shared between workgroups, and its normalised partial output (in T) and
@@ -54,6 +59,8 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   static_assert(DC % 16 == 0 && DC <= D && (PAD || DC == D), "computed head_dim");
   constexpr int KSTEPS = DC / 16;          // contraction steps of QK^T
   constexpr int DBLOCKS = (DC + 31) / 32;  // 32-row blocks of O^T
+  constexpr int kStagePitch = kStagePitchBytes;   // LDS row pitch of the output staging block
+  constexpr int kStageBytes = kStageBytesPerWave;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -308,22 +315,58 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   const float l_tot = sum_halves(l_part);
   const float inv = 1.0f / l_tot;
   const float lse = (m_used * c + fast_log2(l_tot)) * kLn2;
-  if (qrow < p.Sq && (p.acc_out == nullptr || part_out != nullptr)) {
-    T* optr;
-    if (part_out != nullptr) optr = part_out + (wave * kRowsPerWave + l32) * D;
-    else optr = (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
+  if (p.acc_out == nullptr || part_out != nullptr) {
+    // The normalised rows go out through LDS, 64 columns at a time: lane (query, half) writes
+    // its 4-element pieces into a [32 rows][64 columns] block private to the wavefront, which is
+    // read back with 8 lanes per row, so that every global store covers whole 128-byte lines of
+    // 8 rows (stored straight from the accumulator layout, a store touches 32 rows 16 bytes at
+    // a time and the epilogue is bound by the number of memory requests).
+    typedef __attribute__((ext_vector_type(4))) T vec4;
+    __syncthreads();  // every wavefront is done with the fragments of the last tile
+    XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + wave * kStageBytes;
+    const int row0 = qt * kRowsPerBlock + wave * kRowsPerWave;   // first query row of this wavefront
+    T* obase;
+    int64_t ostride;
+    int rows_live = kRowsPerWave;
+    if (part_out != nullptr) {
+      obase = part_out + (int64_t)(wave * kRowsPerWave) * D;
+      ostride = D;
+    } else {
+      obase = (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)row0 * p.os_s;
+      ostride = p.os_s;
+      rows_live = p.Sq - row0;  // may be <= 0 or above 32
+    }
+    const int cols_live = part_out != nullptr ? 32 * DBLOCKS : (PAD ? dact : D);
+    const int rd_row = lane >> 3;          // + 8r
+    const int rd_col = (lane & 7) * 8;     // element column within the 64-column pass
 #pragma unroll
-    for (int db = 0; db < DBLOCKS; db++)
+    for (int half = 0; half < (DBLOCKS + 1) / 2; half++) {
 #pragma unroll
-      for (int a = 0; a < 4; a++) {
-        // registers 4a..4a+3 are d = 32db + 8a + 4hh + 0..3 of this lane's query
-        typedef __attribute__((ext_vector_type(4))) T vec4;
-        f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
-                   oacc[db][4 * a + 3] * inv};
-        vec4 ov = __builtin_convertvector(o, vec4);
-        if (!PAD || part_out != nullptr || 32 * db + 8 * a + 4 * hh < dact) *(vec4*)(optr + 32 * db + 8 * a + 4 * hh) = ov;
+      for (int dbl = 0; dbl < 2; dbl++) {
+        const int db = 2 * half + dbl;
+        if (db < DBLOCKS) {
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            // registers 4a..4a+3 are d = 32db + 8a + 4hh + 0..3 of this lane's query
+            f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                       oacc[db][4 * a + 3] * inv};
+            *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+          }
+        }
       }
-    if (hh == 0) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int row = rd_row + 8 * r;
+        const int col = 64 * half + rd_col;
+        const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
+        if (row < rows_live && col < cols_live) *(vec8*)(obase + row * ostride + col) = x;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (hh == 0 && qrow < p.Sq) {
       if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
       else if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = lse;
     }
@@ -380,7 +423,7 @@ static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 2 : 
 template <typename T, int D, int DC, int NW, bool PAD>
 static hipError_t launch_kernel(const AttnParams& q, hipStream_t stream) {
   static std::atomic<bool> lds_ready[kMaxDevices];
-  constexpr int lds = 2 * TileGeom<D>::BUF_BYTES;
+  constexpr int lds = 2 * TileGeom<D>::BUF_BYTES > NW * kStageBytesPerWave ? 2 * TileGeom<D>::BUF_BYTES : NW * kStageBytesPerWave;
   const int slot = current_device_slot();
   if (!lds_ready[slot].load(std::memory_order_relaxed)) {  // > 64 KiB of dynamic LDS must be enabled once per kernel and device
     hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, DC, NW, PAD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
