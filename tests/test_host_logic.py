@@ -190,3 +190,20 @@ def test_default_backend_by_name():
             usp.set_default_backend("flash_9")
     finally:
         usp.set_default_backend(AB.AttentionBackendType.MI355)
+
+
+def test_bench_refuses_more_than_one_gpu_and_lists_the_model_shapes():
+    """bench.py runs on one GPU only: --gpus above 1 exits with a message before touching a device;
+    the table of model shapes names shapes the kernels accept (head_dim a multiple of 8 up to 128)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout == ""
+    sys.path.insert(0, root)
+    import bench
+    assert len(bench.MODEL_SHAPES) >= 10
+    for name, B, H, Sq, Sk, D in bench.MODEL_SHAPES:
+        assert D % 8 == 0 and 0 < D <= 128 and min(B, H, Sq, Sk) > 0, name
+        assert ops.fused_ring_step_supported(torch.empty(1, 1, 1, D, dtype=torch.bfloat16))
