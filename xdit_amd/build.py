@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJDIR = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libxdit_amd_attn.so")
-SOURCES = ["api.hip", "attn_fwd_16.hip", "attn_fwd_fp8.hip", "attn_fwd_f32.hip", "lse_merge.hip", "fp8_quant.hip", "qk_prologue.hip"]
+SOURCES = ["api.hip", "attn_fwd_16.hip", "attn_fwd_16_ring.hip", "attn_fwd_fp8.hip", "attn_fwd_f32.hip", "lse_merge.hip", "fp8_quant.hip", "qk_prologue.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed-fp32 VALU forms are kept out of the generated code
@@ -45,7 +45,7 @@ def build(verbose=True):
     """Compile every HIP source and link the shared library. Always recompiles."""
     os.makedirs(OBJDIR, exist_ok=True)
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    with ThreadPoolExecutor(max_workers=min(7, len(srcs))) as ex:
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         objs = list(ex.map(_compile, srcs))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)

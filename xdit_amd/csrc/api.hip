@@ -253,7 +253,8 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   hipError_t e;
   if (mfma16_path(a)) {
     p.d_actual = a->D;
-    e = xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a), stream);
+    e = acc != nullptr ? xdit::launch_attn_fwd_16_ring(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a), stream)
+                       : xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a), stream);
   } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
     if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
     e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, rows_per_block_16(a), stream);

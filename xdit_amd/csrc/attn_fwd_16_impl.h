@@ -1,0 +1,526 @@
+// Non-causal attention forward for 16-bit inputs (bf16 / fp16) on gfx950, built for head_dim 64 and 128
+// (tensors of a smaller head_dim, a multiple of 8, run on the next one up: see PAD below).
+//
+// Work decomposition
+//   workgroup = 256 threads = 4 wavefronts; it owns 128 query rows of one (batch, head);
+//   wavefront w owns rows [32w, 32w+32).  Keys/values stream through LDS in tiles of 64 keys,
+//   double buffered, filled by direct global->LDS loads (16 bytes per lane).
+//
+// MFMA orientation (v_mfma_f32_32x32x16_{bf16,f16}; A is 32x16, B is 16x32, lane l holds row/col
+// l%32 and the 8 contraction elements 8*(l/32)..+7; the 32x32 result puts column l%32 and rows
+// 8*(i/4) + 4*(l/32) + i%4, i = 0..15, in lane l):
+//   S^T = K Q^T    A = K tile rows (keys), B = Q^T (kept in registers for the whole kernel)
+//   O^T = V^T P^T  A = V^T (read transposed from LDS with ds_read_b64_tr_b16), B = P^T
+// Computing the transposed products makes every lane own ONE query (column l%32): the softmax
+// row statistics are per-lane scalars (one exchange between the two wavefront halves per tile),
+// and the S^T accumulator registers are, after conversion to 16 bit, exactly the B operand of
+// the second product, so P never goes through LDS.
+//
+// LDS layout: see attn_tiles.h.  The workgroup has NW = 4, 8 or 12 wavefronts (128 / 256 / 384
+// query rows): 8 or 12 wavefronts share every K/V tile, which cuts the L2->LDS traffic per FLOP
+// to a half or a third, and are used when the problem still yields enough workgroups to fill
+// the chip.
+//
+// LDS fragment reads are issued by hand (inline assembly, kPrefetch MFMAs ahead of their use,
+// completion awaited with counted s_waitcnt): left to the compiler, every MFMA waits for a read
+// issued just before it, and the read latency is paid sixteen times per product and tile.
+#pragma once
+#include "attn_split.h"
+#include "launchers.h"
+
+namespace xdit {
+
+constexpr int kRowsPerWave = 32;
+// LDS fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
+constexpr int kPrefetch = 4;
+
+// Output staging block of a wavefront in the epilogue: 32 rows of 64 16-bit columns, rows 8 bytes
+// apart from a multiple of 128 so that the 8-byte writes of the 32 lanes of a half hit 32 banks.
+constexpr int kStagePitchBytes = 64 * 2 + 8;
+constexpr int kStageBytesPerWave = kRowsPerWave * kStagePitchBytes + kRowsPerWave * 4;  // + one fp32 per row (ring step)
+
+// One segment of work: the query tile `tile`, KV tiles [it0, it1).  With `part_out == nullptr` the
+// normalised result goes to the output tensors; otherwise the segment is one PART of a query tile
+// whose KV range is shared between workgroups, and its normalised partial output (in T) and
+// log-sum-exp go to the workspace slot (part_out, part_lse), [row][D] and [row], to be folded by
+// attn_combine_kernel.
+// PAD: the tensors' head_dim (p.d_actual, a multiple of 8) is smaller than D; the missing columns
+// are zeros in the Q fragments and in LDS (cleared here, never written by the tile loads) and are
+// not stored.  DC (a multiple of 16, d_actual <= DC <= D) is the head_dim the two products are
+// computed over: LDS tiles keep the geometry of D, contraction steps (of 16) and output blocks
+// (of 32) past DC are left out.
+template <typename T, int D, int DC, int NW, bool PAD, bool FUSED>
+__device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char* smem, const int tile,
+                                             const int it0, const int it1, T* part_out, float* part_lse) {
+  constexpr int kWaves = NW;
+  constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
+  typedef typename Mfma16<T>::vec8 vec8;
+  typedef typename Mfma16<T>::vec2 vec2;
+  typedef TileGeom<D> G;
+  static_assert(DC % 16 == 0 && DC <= D && (PAD || DC == D), "computed head_dim");
+  constexpr int KSTEPS = DC / 16;          // contraction steps of QK^T
+  constexpr int DBLOCKS = (DC + 31) / 32;  // 32-row blocks of O^T
+  constexpr int kStagePitch = kStagePitchBytes;   // LDS row pitch of the output staging block
+  constexpr int kStageBytes = kStageBytesPerWave;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  const int bh = tile / p.nq_tiles;
+  const int qt = tile - bh * p.nq_tiles;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+
+  // ---- Q fragments: B operand of S^T, lane = (query l32, contraction half hh) -------------
+  const int qrow = qt * kRowsPerBlock + wave * kRowsPerWave + l32;
+  const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
+  const T* qptr = (const T*)p.q + b * p.qs_b + h * p.qs_h + (int64_t)qrow_c * p.qs_s + hh * 8;
+  const int dact = PAD ? p.d_actual : D;
+  vec8 qf[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ks++) {
+    if (!PAD || ks * 16 + hh * 8 < dact) {
+      qf[ks] = *(const vec8*)(qptr + ks * 16);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) qf[ks][e] = (T)0.f;
+    }
+  }
+
+  // ---- direct global->LDS tile loads ------------------------------------------------------
+  // A tile is 2*NG pieces of 1 KiB (K pieces 0..NG-1, then V pieces): piece g of K (or V) holds
+  // rows g, g+NG, g+2NG, ...; wavefront w loads pieces w, w+NW, w+2NW, ...; within a piece
+  // lane -> (slot = lane / lanes-per-row, 16-byte column = lane % lanes-per-row).  A load is
+  // "uniform 64-bit tile base + per-lane 32-bit byte offset".
+  const T* kbase1 = (const T*)p.k + b * p.ks_b + h * p.ks_h;
+  const T* vbase1 = (const T*)p.v + b * p.vs_b + h * p.vs_h;
+  const T* kbase2 = p.Sk2 > 0 ? (const T*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
+  const T* vbase2 = p.Sk2 > 0 ? (const T*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
+  constexpr int LANES_PER_ROW = G::ROW_BYTES / 16;
+  // Loader wavefronts: the first LW wavefronts each load PAIRS (K piece g, V piece g) pairs,
+  // g = wave + LW * i, with one row index per lane for both pieces of a pair.
+  constexpr int LW = kWaves < 8 ? kWaves : 8;
+  constexpr int PAIRS = G::NG / LW;
+  static_assert(G::NG % LW == 0, "pieces must divide evenly over the loader wavefronts");
+  const int ld_row0 = G::NG * (lane / LANES_PER_ROW) + wave;  // row of this lane in pair 0
+  const unsigned ld_colb = (lane % LANES_PER_ROW) * 16;       // byte offset inside the row
+  const bool ld_on = !PAD || ld_colb < (unsigned)dact * 2;    // lanes of columns the tensors do not have stay idle
+  const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS unsigned char*)smem;
+  const unsigned ld_kdst = lds_base + wave * G::K_PITCH;      // LDS address of K piece `wave`, buffer 0
+  const unsigned ld_vdst = lds_base + G::K_BYTES + wave * G::V_PITCH;
+
+  const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
+  const int nt2 = (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  const int nt = nt1 + nt2;
+
+  // Stream position: base pointers of the next tile to load, byte strides, keys left in its segment.
+  const T* ld_kp;
+  const T* ld_vp;
+  unsigned ld_kss, ld_vss;
+  int64_t ld_kstep, ld_vstep;
+  int ld_left;
+  auto seek_tile = [&](int t) {
+    if (t < nt1) {
+      ld_kp = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
+      ld_vp = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
+      ld_kss = (unsigned)(p.ks_s * 2); ld_vss = (unsigned)(p.vs_s * 2);
+      ld_kstep = kKeysPerTile * p.ks_s; ld_vstep = kKeysPerTile * p.vs_s;
+      ld_left = p.Sk - t * kKeysPerTile;
+    } else {
+      ld_kp = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
+      ld_vp = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
+      ld_kss = (unsigned)(p.k2s_s * 2); ld_vss = (unsigned)(p.v2s_s * 2);
+      ld_kstep = kKeysPerTile * p.k2s_s; ld_vstep = kKeysPerTile * p.v2s_s;
+      ld_left = p.Sk2 - (t - nt1) * kKeysPerTile;
+    }
+  };
+  // Loads the tile at the stream position into buffer `buf` and advances the position.
+  auto issue_tile = [&](int t, int buf) {
+    if ((kWaves == LW || wave < LW) && ld_on) {
+      const int last = (ld_left < kKeysPerTile ? ld_left : kKeysPerTile) - 1;
+      const unsigned bo = buf * G::BUF_BYTES;
+#pragma unroll
+      for (int i = 0; i < PAIRS; i++) {
+        int r = ld_row0 + LW * i;
+        r = r < last ? r : last;  // rows past the end of the segment re-read its last row
+        load_lds_16(ld_kp, __umul24((unsigned)r, ld_kss) + ld_colb, ld_kdst + bo + i * LW * G::K_PITCH);
+        load_lds_16(ld_vp, __umul24((unsigned)r, ld_vss) + ld_colb, ld_vdst + bo + i * LW * G::V_PITCH);
+      }
+    }
+    if (t + 1 == nt1) {
+      seek_tile(t + 1);
+    } else {
+      ld_kp += ld_kstep; ld_vp += ld_vstep; ld_left -= kKeysPerTile;
+    }
+  };
+
+  // ---- LDS read addresses: one per-lane base each for K and V, the rest are immediates ------
+  // K fragment (A operand of S^T) for key block kb, step ks: row 32kb + l32, bytes 32ks + 16hh.
+  //   row -> piece (row % NG), slot (row / NG)
+  const int kbase_off = (l32 % G::NG) * G::K_PITCH + (l32 / G::NG) * G::ROW_BYTES + hh * 16;
+  constexpr int K_KB_STEP = (32 / G::NG) * G::ROW_BYTES;  // +32 rows = +32/NG slots
+  // V^T fragment (A operand of O^T) for d block db, key step j (16 keys), half rd (keys +0 / +8):
+  // as a SOURCE lane of the transposed read, lane (group g = lane/16, s = lane%16) supplies the
+  // 8 bytes at key row 16j + 8rd + 4hh + s/4, elements d = 32db + 16(g%2) + 4(s%4) .. +3; the
+  // read returns to lane (g, i) the four keys of that row group at d = 32db + 16(g%2) + i.
+  const int vsrc_row = 4 * hh + ((lane & 15) >> 2);  // row within the 16-key step, rd = 0
+  const int vbase_off = (vsrc_row % G::NG) * G::V_PITCH + (vsrc_row / G::NG) * G::ROW_BYTES +
+                        (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  // +8 rows (rd) and +16 rows (j): both keep row % NG pattern simple because NG is 8 or 16.
+  constexpr int V_RD_STEP = (G::NG == 16) ? 8 * G::V_PITCH : G::ROW_BYTES;  // NG=8: +8 rows = +1 slot
+  constexpr int V_J_STEP = (16 / G::NG) * G::ROW_BYTES;
+
+  // ---- online softmax state: one query per lane (both halves of the wavefront agree) ------
+  const float c = p.scale * kLog2e;  // logits are kept in log2 units
+  float m_used = -INFINITY;          // running (lazily updated) row maximum of the raw dot products
+  float l_part = 0.f;                // this lane's share of the running row sum
+  f32x16 oacc[DBLOCKS];
+#pragma unroll
+  for (int db = 0; db < DBLOCKS; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+
+  if (PAD) {  // zero the columns that no load writes (all of both buffers: simplest)
+    typedef __attribute__((ext_vector_type(4))) int i32x4;
+    const i32x4 zero = {0, 0, 0, 0};
+    for (int i = tid * 16; i < 2 * G::BUF_BYTES; i += 64 * kWaves * 16) *(XDIT_LDS i32x4*)((XDIT_LDS unsigned char*)smem + i) = zero;
+    __syncthreads();
+  }
+  seek_tile(it0);
+  issue_tile(it0, 0);
+  // Make the compiler account for the Q fragment loads here, before the loop: the tile loads
+  // above are invisible to its outstanding-load bookkeeping, so any wait it placed for a Q
+  // fragment inside the loop would also wait for the prefetch of the next tile.
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+v"(qf[ks]));
+
+  for (int t = it0; t < it1; t++) {
+    const int buf = (t - it0) & 1;
+    // Tile t has landed (this thread's loads) and, after the barrier, everyone's; the barrier
+    // also means every wavefront is done reading the other buffer, which tile t+1 now overwrites.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (t + 1 < it1) issue_tile(t + 1, buf ^ 1);
+
+    const XDIT_LDS unsigned char* ktile =
+        (const XDIT_LDS unsigned char*)(smem + buf * G::BUF_BYTES) + kbase_off;
+    const XDIT_LDS unsigned char* vtile =
+        (const XDIT_LDS unsigned char*)(smem + buf * G::BUF_BYTES + G::K_BYTES) + vbase_off;
+
+    // ---- S^T = K Q^T : 2 blocks of 32 keys x 32 queries ---------------------------------
+    f32x16 sacc[2];
+    {
+      constexpr int PD = kPrefetch;   // K fragment reads in flight
+      constexpr int NR = 2 * KSTEPS;  // reads (= MFMAs) of this product
+      const unsigned kaddr = (unsigned)(uintptr_t)ktile;
+      vec8 kf[NR];
+      static_for<PD>([&](auto I) {
+        constexpr int i = I;
+        lds_read_b128<(i / KSTEPS) * K_KB_STEP + (i % KSTEPS) * 32>(kf[i], kaddr);
+      });
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+      static_for<NR>([&](auto I) {
+        constexpr int i = I;
+        constexpr int younger = (i + PD <= NR ? PD : NR - i) - 1;
+        lds_wait<younger>(kf[i]);
+        sacc[i / KSTEPS] = Mfma16<T>::mma(kf[i], qf[i % KSTEPS], sacc[i / KSTEPS]);
+        if constexpr (i + PD < NR) {
+          constexpr int n = i + PD;
+          lds_read_b128<(n / KSTEPS) * K_KB_STEP + (n % KSTEPS) * 32>(kf[n], kaddr);
+        }
+      });
+    }
+    // ---- mask keys past the end of the segment (only its last tile can be partial) -------
+    const int valid = (t < nt1) ? p.Sk - t * kKeysPerTile : p.Sk2 - (t - nt1) * kKeysPerTile;
+    if (valid < kKeysPerTile) {
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          int key = 32 * kb + 8 * (i >> 2) + 4 * hh + (i & 3);
+          if (key >= valid) sacc[kb][i] = -INFINITY;
+        }
+    }
+
+    // ---- online softmax ---------------------------------------------------------------
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[0][i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[1][i]);
+    mx = max_halves(mx);
+    const float m_new = fmaxf(m_used, mx);
+    const bool grow = (m_new - m_used) * c > kLazyRescaleLog2;  // true on the first tile (-inf)
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float alpha = fast_exp2((m_used - m_new) * c);  // 0 on the first tile
+      m_used = m_new;
+      l_part *= alpha;
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+    }
+    const float mc = m_used * c;
+    vec8 pf[4];  // P^T as B operands: pf[j] = keys 16j..16j+15 of this tile (permuted inside)
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        float p0 = fast_exp2(__builtin_fmaf(sacc[kb][i], c, -mc));
+        float p1 = fast_exp2(__builtin_fmaf(sacc[kb][i + 1], c, -mc));
+        l_part += p0 + p1;
+        f32x2 pp = {p0, p1};
+        vec2 pk = __builtin_convertvector(pp, vec2);
+        const int j = 2 * kb + (i >> 3);
+        pf[j][(i & 7)] = pk[0];
+        pf[j][(i & 7) + 1] = pk[1];
+      }
+    }
+
+    // ---- O^T += V^T P^T ------------------------------------------------------------------
+    {
+      constexpr int PD = kPrefetch;  // MFMAs whose two V^T reads are in flight
+      constexpr int NM = 4 * DBLOCKS;
+      typedef __attribute__((ext_vector_type(8))) short s16x8;
+      const unsigned vaddr = (unsigned)(uintptr_t)vtile;
+      s16x4 v0[NM], v1[NM];
+      static_for<PD>([&](auto I) {
+        constexpr int i = I;
+        constexpr int off = (i / DBLOCKS) * V_J_STEP + (i % DBLOCKS) * 64;
+        lds_read_tr16_b64<off>(v0[i], vaddr);
+        lds_read_tr16_b64<off + V_RD_STEP>(v1[i], vaddr);
+      });
+      static_for<NM>([&](auto I) {
+        constexpr int i = I;
+        constexpr int younger = 2 * ((i + PD <= NM ? PD : NM - i) - 1);
+        lds_wait2<younger>(v0[i], v1[i]);
+        s16x8 vv = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        oacc[i % DBLOCKS] = Mfma16<T>::mma(__builtin_bit_cast(vec8, vv), pf[i / DBLOCKS], oacc[i % DBLOCKS]);
+        if constexpr (i + PD < NM) {
+          constexpr int n = i + PD;
+          constexpr int off = (n / DBLOCKS) * V_J_STEP + (n % DBLOCKS) * 64;
+          lds_read_tr16_b64<off>(v0[n], vaddr);
+          lds_read_tr16_b64<off + V_RD_STEP>(v1[n], vaddr);
+        }
+      });
+    }
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------
+  const float l_tot = sum_halves(l_part);
+  const float inv = 1.0f / l_tot;
+  const float lse = (m_used * c + fast_log2(l_tot)) * kLn2;
+  if constexpr (!FUSED) {
+    // The normalised rows go out through LDS, 64 columns at a time: lane (query, half) writes
+    // its 4-element pieces into a [32 rows][64 columns] block private to the wavefront, which is
+    // read back with 8 lanes per row, so that every global store covers whole 128-byte lines of
+    // 8 rows (stored straight from the accumulator layout, a store touches 32 rows 16 bytes at
+    // a time and the epilogue is bound by the number of memory requests).
+    typedef __attribute__((ext_vector_type(4))) T vec4;
+    __syncthreads();  // every wavefront is done with the fragments of the last tile
+    XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + wave * kStageBytes;
+    const int row0 = qt * kRowsPerBlock + wave * kRowsPerWave;   // first query row of this wavefront
+    T* obase;
+    int64_t ostride;
+    int rows_live = kRowsPerWave;
+    if (part_out != nullptr) {
+      obase = part_out + (int64_t)(wave * kRowsPerWave) * D;
+      ostride = D;
+    } else {
+      obase = (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)row0 * p.os_s;
+      ostride = p.os_s;
+      rows_live = p.Sq - row0;  // may be <= 0 or above 32
+    }
+    const int cols_live = part_out != nullptr ? 32 * DBLOCKS : (PAD ? dact : D);
+    const int rd_row = lane >> 3;          // + 8r
+    const int rd_col = (lane & 7) * 8;     // element column within the 64-column pass
+#pragma unroll
+    for (int half = 0; half < (DBLOCKS + 1) / 2; half++) {
+#pragma unroll
+      for (int dbl = 0; dbl < 2; dbl++) {
+        const int db = 2 * half + dbl;
+        if (db < DBLOCKS) {
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            // registers 4a..4a+3 are d = 32db + 8a + 4hh + 0..3 of this lane's query
+            f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                       oacc[db][4 * a + 3] * inv};
+            *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int row = rd_row + 8 * r;
+        const int col = 64 * half + rd_col;
+        const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
+        if (row < rows_live && col < cols_live) *(vec8*)(obase + row * ostride + col) = x;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (hh == 0 && qrow < p.Sq) {
+      if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
+      else if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = lse;
+    }
+  } else {
+    // Ring step: fold this block into the fp32 accumulator (the arithmetic of the merge kernel
+    // on the block rounded to T, so the result equals forward + merge bit for bit).  The block
+    // goes through the same LDS transpose as above, so that the accumulator is read and written
+    // in whole rows; the weight of each row's fold travels with it.
+    typedef __attribute__((ext_vector_type(4))) T vec4;
+    __syncthreads();  // every wavefront is done with the fragments of the last tile
+    XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + wave * kStageBytes;
+    XDIT_LDS float* wrow = (XDIT_LDS float*)(stage + kRowsPerWave * kStagePitch);
+    const int row0 = qt * kRowsPerBlock + wave * kRowsPerWave;
+    const bool first = p.acc_first != 0;
+    float* alp = p.acc_lse + b * p.al_b + h * p.al_h + (int64_t)qrow * p.al_s;
+    float w = 0.f, new_lse = lse;
+    if (!first && qrow < p.Sq) {
+      const float la = *alp;
+      w = sigmoid(lse - la);
+      new_lse = la - log_sigmoid(la - lse);
+    }
+    if (hh == 0) wrow[l32] = w;
+    float* abase = p.acc_out + b * p.ao_b + h * p.ao_h + (int64_t)row0 * p.ao_s;
+    T* obase = p.out != nullptr ? (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)row0 * p.os_s : nullptr;
+    const int rows_live = p.Sq - row0;
+    const int cols_live = PAD ? dact : D;
+    const int rd_row = lane >> 3;
+    const int rd_col = (lane & 7) * 8;
+#pragma unroll
+    for (int half = 0; half < (DBLOCKS + 1) / 2; half++) {
+#pragma unroll
+      for (int dbl = 0; dbl < 2; dbl++) {
+        const int db = 2 * half + dbl;
+        if (db < DBLOCKS) {
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                       oacc[db][4 * a + 3] * inv};
+            *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int row = rd_row + 8 * r;
+        const int col = 64 * half + rd_col;
+        const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
+        const float wr = wrow[row];
+        if (row < rows_live && col < cols_live) {
+          float* aptr = abase + row * p.ao_s + col;
+          f32x4 m0, m1;
+#pragma unroll
+          for (int e = 0; e < 4; e++) { m0[e] = (float)x[e]; m1[e] = (float)x[4 + e]; }
+          if (!first) {
+            const f32x4 a0 = *(const f32x4*)aptr, a1 = *(const f32x4*)(aptr + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) { m0[e] = fold_value(a0[e], m0[e], wr); m1[e] = fold_value(a1[e], m1[e], wr); }
+          }
+          if (p.acc_store) { *(f32x4*)aptr = m0; *(f32x4*)(aptr + 4) = m1; }
+          if (obase != nullptr) {
+            vec8 y;
+#pragma unroll
+            for (int e = 0; e < 4; e++) { y[e] = (T)m0[e]; y[4 + e] = (T)m1[e]; }
+            *(vec8*)(obase + row * p.os_s + col) = y;
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (hh == 0 && qrow < p.Sq) {
+      *alp = new_lse;
+      if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = new_lse;
+    }
+  }
+}
+
+template <typename T, int D, int DC, int NW, bool PAD, bool FUSED>
+__global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(const AttnParams p) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // 2 x [K tile | V tile]
+  run_workgroup<T, kRowsPerWave * NW, D>(p, [&](int tile, int it0, int it1, T* part_out, float* part_lse) {
+    attn_segment<T, D, DC, NW, PAD, FUSED>(p, smem, tile, it0, it1, part_out, part_lse);
+  });
+}
+
+// Workgroups of NW wavefronts resident at once: LDS and registers allow two 4-wavefront
+// workgroups per CU, one otherwise.
+static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 2 : 1); }
+
+template <typename T, int D, int DC, int NW, bool PAD, bool FUSED>
+static hipError_t launch_kernel(const AttnParams& q, hipStream_t stream) {
+  static std::atomic<bool> lds_ready[kMaxDevices];
+  constexpr int lds = 2 * TileGeom<D>::BUF_BYTES > NW * kStageBytesPerWave ? 2 * TileGeom<D>::BUF_BYTES : NW * kStageBytesPerWave;
+  const int slot = current_device_slot();
+  if (!lds_ready[slot].load(std::memory_order_relaxed)) {  // > 64 KiB of dynamic LDS must be enabled once per kernel and device
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, DC, NW, PAD, FUSED>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    lds_ready[slot].store(true, std::memory_order_relaxed);
+  }
+  hipLaunchKernelGGL((attn_fwd_16_kernel<T, D, DC, NW, PAD, FUSED>), dim3(split_grid(q)), dim3(64 * NW), lds, stream, q);
+  return hipSuccess;
+}
+
+template <typename T, int D, int NW, bool FUSED>
+static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
+  AttnParams q = p;
+  constexpr int rows = 32 * NW;
+  q.nq_tiles = (p.Sq + rows - 1) / rows;
+  q.total_tiles = p.B * p.H * q.nq_tiles;
+  q.tiles_per_xcd = (q.total_tiles + 7) / 8;
+  // the ring step folds in the epilogue of whole query tiles: no shared last round
+  bind_workspace(q, p, FUSED ? 0 : plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup), rows, D, 2);
+  if constexpr (!FUSED) {
+    if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
+  }
+  if (q.d_actual == D) q.d_actual = 0;
+  // computed head_dims built for tensors smaller than D: 80, 96, 112 (and 128) of 128; 32 (and 64) of 64
+  hipError_t e;
+  if (q.d_actual == 0) {
+    e = launch_kernel<T, D, D, NW, false, FUSED>(q, stream);
+  } else if constexpr (D == 128) {
+    e = q.d_actual <= 80    ? launch_kernel<T, D, 80, NW, true, FUSED>(q, stream)
+        : q.d_actual <= 96  ? launch_kernel<T, D, 96, NW, true, FUSED>(q, stream)
+        : q.d_actual <= 112 ? launch_kernel<T, D, 112, NW, true, FUSED>(q, stream)
+                            : launch_kernel<T, D, 128, NW, true, FUSED>(q, stream);
+  } else {
+    e = q.d_actual <= 32 ? launch_kernel<T, D, 32, NW, true, FUSED>(q, stream) : launch_kernel<T, D, 64, NW, true, FUSED>(q, stream);
+  }
+  if (e != hipSuccess) return e;
+  if constexpr (!FUSED) {
+    if (q.split_units) {
+      const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+      const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
+      hipLaunchKernelGGL((attn_combine_kernel<T, D>), cgrid, dim3(256), 0, stream, q, rows, nt);
+    }
+  }
+  return hipGetLastError();
+}
+
+// D: the head_dim the kernel is built for, 128 or 64; p.d_actual, if not 0, is the tensors'
+// smaller head_dim (a multiple of 8).  rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12).
+// FUSED: the ring step (p.acc_out set), whose epilogue folds the block into the accumulator.
+template <typename T, bool FUSED>
+static hipError_t launch_typed(const AttnParams& p, int D, int rows_per_block, hipStream_t stream) {
+  if (D == 128 && rows_per_block == 384) return launch_one<T, 128, 12, FUSED>(p, stream);
+  if (D == 128 && rows_per_block == 256) return launch_one<T, 128, 8, FUSED>(p, stream);
+  if (D == 128) return launch_one<T, 128, 4, FUSED>(p, stream);
+  if (D == 64 && rows_per_block == 384) return launch_one<T, 64, 12, FUSED>(p, stream);
+  if (D == 64 && rows_per_block == 256) return launch_one<T, 64, 8, FUSED>(p, stream);
+  if (D == 64) return launch_one<T, 64, 4, FUSED>(p, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace xdit

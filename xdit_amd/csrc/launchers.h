@@ -68,6 +68,7 @@ struct PrologueBatch {
 
 // dtype codes below are the C ABI's xdit_dtype values: 0 bf16, 1 fp16, 2 fp32, 3 fp8 e4m3fn.
 hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream);
+hipError_t launch_attn_fwd_16_ring(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream);  // p.acc_out set
 size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block, AttnParams* plan = nullptr);
 hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream);
 size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan = nullptr);
