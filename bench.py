@@ -242,7 +242,7 @@ def main():
             also["c2_flux1024_torch_flash_same_gpu"] = {"error": str(e)[:120]}
         # ring of 4 KV chunks, merged in fp32 (the cast of the last fold is fused)
         fn = usp._get_attention_function()
-        _, ms = time_calls(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), n, 3)
+        _, ms = time_calls(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), max(n, args.steps // 4), args.warmup)
         also["c3_flux_ring4"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
         # the same ring captured once in a HIP graph and replayed (shows whether the eager form is launch-bound)
         side = torch.cuda.Stream()
@@ -254,7 +254,7 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             usp.ring_attn(fn, q, k, v, ring_chunks=4)
-        _, ms = time_calls(graph.replay, n, 3)
+        _, ms = time_calls(graph.replay, max(n, args.steps // 4), args.warmup)
         also["c3_flux_ring4_graph"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
         del graph
         # the merge kernel alone: bytes per fold = 10*N*D + 12*N
