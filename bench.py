@@ -38,7 +38,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-MEASURED_HBM_BYTES_PER_LAUNCH = 201.6e6  # Flux-1024 bf16 step: 147.3 MB read + 54.3 MB written (attention + combine kernels)
+MEASURED_HBM_BYTES_PER_LAUNCH = 211.1e6  # Flux-1024 bf16 step: 153.6 MB read + 57.5 MB written (attention + combine kernels)
 
 
 def make_inputs(B, H, S, D, seed, device, rmsnorm=True, dtype=torch.bfloat16):
@@ -217,7 +217,7 @@ def main():
             # HBM bytes per step from rocprofv3 FETCH_SIZE / WRITE_SIZE counters, each scaled by the
             # same counter's reading for a 256 MiB copy in the same run (--copy-calibration)
             "traffic": MEASURED_HBM_BYTES_PER_LAUNCH,
-            "kernel": "attn_fwd_16_kernel<bf16,128,128,12,false> (+ attn_combine_kernel<bf16,128> for the shared last round)",
+            "kernel": "attn_fwd_16_kernel<bf16,128,128,12,false,false> (+ attn_combine_kernel<bf16,128> for the shared last round)",
             "kernel_ms": round(ev_ms, 5),
         },
     }
