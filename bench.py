@@ -17,7 +17,12 @@ q/k per-head RMSNorm'd), inputs resident in HBM.  Prints ONE JSON line:
                shard (fp8), the 4-chunk ring with its fp32 merges, the merge kernel's GB/s, the
                fp8 quantiser and the fused norm + rotary prologue (GB/s against the HBM peak)
                and torch's own GPU flash attention (the op behind the reference's default
-               SDPA_FLASH backend, attention_backend.py:504-516) on the same tensors and GPU
+               SDPA_FLASH backend, attention_backend.py:504-516) on the same tensors and GPU;
+               the PixArt-512 fp32 case; the Flux step's first 25 calls and its steady state in a
+               fresh process (per-call HIP-event pairs: median and min); host time per call
+  Entries of `also` carry the median ("ms" / "us"), the minimum and the mean of per-call
+  HIP-event pairs (the reference times its own runs with events around synchronised regions
+  and discards the first iteration: xfuser/model_executor/models/runner_models/base_model.py:631-644).
 --model-shapes prints, instead of the JSON line, one row per attention shape of the reference's
 model families (self, joint and cross attention; head_dim 128, 64, 72, 88): this library against
 torch's GPU flash attention on the same tensors, with the largest difference between the outputs.
@@ -37,8 +42,22 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-MEASURED_HBM_BYTES_PER_LAUNCH = 211.1e6  # Flux-1024 bf16 step: 153.6 MB read + 57.5 MB written (attention + combine kernels)
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "attn_fwd_bf16_flux1024_hbm_traffic.md")
+
+
+def measured_traffic():
+    """HBM bytes per Flux-1024 step as the committed counter summary states them (a line
+    `traffic_bytes_per_step: N` plus the commit the counters were taken at); None if absent."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, None
+    import re
+    m = re.search(r"^traffic_bytes_per_step:\s*([0-9.eE+]+)", text, re.M)
+    c = re.search(r"^measured_at_commit:\s*(\S+)", text, re.M)
+    return (float(m.group(1)) if m else None), (c.group(1) if c else None)
 
 
 def make_inputs(B, H, S, D, seed, device, rmsnorm=True, dtype=torch.bfloat16):
@@ -71,6 +90,60 @@ def time_calls(fn, steps, warmup):
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+
+def time_each(fn, steps, warmup):
+    """Per-call HIP-event pairs on the current stream -> dict(ms median, ms_min, ms_mean)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    t = sorted(a.elapsed_time(b) for a, b in ev)
+    return {"ms": round(t[len(t) // 2], 5), "ms_min": round(t[0], 5), "ms_mean": round(sum(t) / len(t), 5)}
+
+
+def host_us_per_call(fn, batch=40, repeats=5):
+    """Host time of a call that only queues work: `batch` calls back to back without waiting for
+    the GPU, smallest per-call average over `repeats` batches (the queue is drained in between)."""
+    best = None
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(batch):
+            fn()
+        t = (time.perf_counter() - t0) / batch
+        best = t if best is None or t < best else best
+    torch.cuda.synchronize()
+    return round(best * 1e6, 2)
+
+
+def with_rate(stat, flops, peak=None):
+    stat = dict(stat)
+    stat["tflops"] = round(flops / stat["ms"] / 1e9, 1)
+    if peak:
+        stat["frac_peak"] = round(flops / stat["ms"] / 1e9 / peak, 4)
+    return stat
+
+
+def series(dev, calls):
+    """Per-call HIP-event times (us) of the first `calls` Flux-1024 steps of this process."""
+    from xdit_amd import ops
+    q, k, v = make_inputs(1, 24, 4608, 128, 1002, dev)
+    out = torch.empty_like(q)
+    lse = torch.empty(1, 24, 4608, dtype=torch.float32, device=dev)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(calls)]
+    for a, b in ev:
+        a.record()
+        ops.attn_fwd(q, k, v, out=out, lse=lse)
+        b.record()
+    torch.cuda.synchronize()
+    print(json.dumps([round(a.elapsed_time(b) * 1e3, 1) for a, b in ev]))
 
 
 def attn_flops(B, H, Sq, Sk, D):
@@ -123,31 +196,58 @@ def model_shapes(dev):
         del q, k, v, o
 
 
-def cpu_baseline(q, k, v, budget_s=12.0):
-    """The reference's CPU SDPA path on the same Flux-1024 tensors (all heads, fp32), repeated
-    for about `budget_s` seconds of CPU work; reports the median run."""
-    from oracle import attn_oracle as O   # the checker/baseline module; never used by the GPU leg
-    B, H, S, D = q.shape
-    qc, kc, vc = (t.float().cpu().contiguous() for t in (q, k, v))
-    O.sdpa_cpu(qc[:, :1], kc[:, :1], vc[:, :1])  # warm the thread pool
+def _median_time(fn, budget_s, max_runs):
     times = []
     t_start = time.perf_counter()
     while True:
         t0 = time.perf_counter()
-        O.sdpa_cpu(qc, kc, vc)
+        fn()
         times.append(time.perf_counter() - t0)
-        if time.perf_counter() - t_start > budget_s or len(times) >= 200:
+        if time.perf_counter() - t_start > budget_s or len(times) >= max_runs:
             break
-    t = sorted(times)[len(times) // 2]
+    return sorted(times)[len(times) // 2], len(times)
+
+
+def cpu_baseline(q, k, v, budget_s=8.0):
+    """The reference's CPU SDPA path (torch CPU scaled_dot_product_attention, the call inside its
+    SDPA adapter) on this host's cores.  Headline figure: the same Flux-1024 tensors, all heads,
+    fp32, median of full-shape runs over about `budget_s` seconds.  `others`: the same tensors in
+    bf16, PixArt-512 in fp32 at full shape, and for the two video shards the first 2048 query
+    rows against the full keys/values (measured) with the linear-in-Sq figure for the whole
+    shard next to it, labelled as extrapolated."""
+    from oracle import attn_oracle as O   # the checker/baseline module; never used by the GPU leg
+    B, H, S, D = q.shape
+    qc, kc, vc = (t.float().cpu().contiguous() for t in (q, k, v))
+    O.sdpa_cpu(qc[:, :1], kc[:, :1], vc[:, :1])  # warm the thread pool
+    t, runs = _median_time(lambda: O.sdpa_cpu(qc, kc, vc), budget_s, 200)
+    others = {}
+    qb, kb, vb = (x.bfloat16() for x in (qc, kc, vc))
+    tb, rb = _median_time(lambda: O.sdpa_cpu(qb, kb, vb), 3.0, 50)
+    others["c2_flux1024_bf16"] = {"s": round(tb, 4), "tflops": round(attn_flops(B, H, S, S, D) / tb / 1e12, 4), "runs": rb}
+    g = torch.Generator().manual_seed(1001)
+    q1, k1, v1 = (torch.randn(1, 16, 1024, 72, generator=g) for _ in range(3))
+    t1, r1 = _median_time(lambda: O.sdpa_cpu(q1, k1, v1), 1.5, 200)
+    others["c1_pixart512_fp32"] = {"s": round(t1, 5), "tflops": round(attn_flops(1, 16, 1024, 1024, 72) / t1 / 1e12, 4), "runs": r1}
+    for name, (Hs, Ss) in (("c4_hunyuan720p_shard", (3, 118800 + 256)), ("c5_wan720p_shard_dequantised_fp32", (5, 75600))):
+        rows = 2048
+        qs = torch.randn(1, Hs, rows, D, generator=g)
+        ks, vs = (torch.randn(1, Hs, Ss, D, generator=g) for _ in range(2))
+        ts, rs = _median_time(lambda: O.sdpa_cpu(qs, ks, vs), 2.0, 5)
+        others[name] = {"q_rows_measured": rows, "s_measured": round(ts, 4),
+                        "tflops": round(attn_flops(1, Hs, rows, Ss, D) / ts / 1e12, 4),
+                        "s_whole_shard_extrapolated": round(ts * Ss / rows, 2), "runs": rs,
+                        "note": "fp32, first 2048 query rows x all keys of every shard head; whole-shard time is linear-in-Sq extrapolation, not measured"}
+        del qs, ks, vs
     return {
         "value": round(attn_flops(B, H, S, S, D) / t / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": "torch CPU scaled_dot_product_attention (the call inside the reference's SDPA adapter), fp32 copies of "
-                  "the same Flux-1024 tensors (B=1, H=%d, S=%d, D=%d), median of %d full-shape runs over %.1f s, "
+                  "the same Flux-1024 tensors (B=1, H=%d, S=%d, D=%d), median of %d full-shape runs, "
                   "%.3f s per run; host has %d logical CPUs, torch uses %d threads"
-                  % (H, S, D, len(times), time.perf_counter() - t_start, t, os.cpu_count(), torch.get_num_threads()),
+                  % (H, S, D, runs, t, os.cpu_count(), torch.get_num_threads()),
+        "others": others,
     }
 
 
@@ -160,6 +260,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--model-shapes", action="store_true",
                     help="print a table of the reference's model shapes against torch's GPU flash attention, and exit")
+    ap.add_argument("--series", type=int, default=0,
+                    help="print the per-call HIP-event times (us) of the first N Flux-1024 steps of this process, and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof byte counters)")
     args = ap.parse_args()
@@ -178,6 +280,9 @@ def main():
     if args.model_shapes:
         model_shapes(dev)
         return
+    if args.series:
+        series(dev, args.series)
+        return
     B, H, S, D = 1, 24, 4608, 128
     q, k, v = make_inputs(B, H, S, D, 1002, dev)
     out = torch.empty_like(q)
@@ -190,6 +295,7 @@ def main():
     tflops = flops / (wall_ms * 1e-3) / 1e12
     achieved = flops / (ev_ms * 1e-3) / 1e12
 
+    traffic, traffic_commit = measured_traffic()
     result = {
         "metric": "joint-attn fwd ms/call + TFLOP/s (% MFMA peak) at Flux-1024 and HV-720p shard",
         "value": round(tflops, 2),
@@ -216,7 +322,8 @@ def main():
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
             # HBM bytes per step from rocprofv3 FETCH_SIZE / WRITE_SIZE counters, each scaled by the
             # same counter's reading for a 256 MiB copy in the same run (--copy-calibration)
-            "traffic": MEASURED_HBM_BYTES_PER_LAUNCH,
+            "traffic": traffic,
+            "traffic_source": "profiles/attn_fwd_bf16_flux1024_hbm_traffic.md, counters taken at commit %s" % traffic_commit,
             "kernel": "attn_fwd_16_kernel<bf16,128,128,12,false,false> (+ attn_combine_kernel<bf16,128> for the shared last round)",
             "kernel_ms": round(ev_ms, 5),
         },
@@ -224,26 +331,48 @@ def main():
 
     if not args.no_extras:
         also = {}
-        n = max(5, args.steps // 10)
+        n = max(20, args.steps)
+        # The Flux step in a fresh process, per call: the first 25 calls and the steady state
+        # (calls 101..300).  The first few dozen calls after start-up run slower than the steady
+        # state (the chip's power management settles), which is where a short timed window lies.
+        try:
+            import subprocess
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--series", "300"], capture_output=True, text=True, timeout=300)
+            us = json.loads(r.stdout.strip().splitlines()[-1])
+            first, steady = sorted(us[:25]), sorted(us[100:])
+            also["c2_flux1024_first25"] = {"us": first[len(first) // 2], "us_min": first[0], "us_max": first[-1],
+                                           "us_mean": round(sum(first) / len(first), 1), "calls": "1-25 of a fresh process"}
+            also["c2_flux1024_steady"] = {"us": steady[len(steady) // 2], "us_min": steady[0], "us_max": steady[-1],
+                                          "us_mean": round(sum(steady) / len(steady), 1), "calls": "101-300 of the same process",
+                                          "tflops": round(flops / steady[len(steady) // 2] / 1e6, 1),
+                                          "frac_peak": round(flops / steady[len(steady) // 2] / 1e6 / PEAK_BF16_TFLOPS, 4)}
+        except Exception as e:  # the series is a report, not a gate
+            also["c2_flux1024_first25"] = {"error": str(e)[:160]}
+        # host time of the calls (the Python wrapper + the C entry point; nothing waits for the GPU)
+        lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
+        also["host_us_per_call"] = {"attn_fwd": host_us_per_call(lambda: ops.attn_fwd(q, k, v, out=out, lse=lse)),
+                                    "attn_fwd_allocating_out_and_lse": host_us_per_call(lambda: ops.attn_fwd(q, k, v))}
         # the plain launch (one workgroup per query tile, no shared last round, no combine kernel)
-        # (these two are timed like the headline: a shape's first few dozen calls run slower)
-        _, ms = time_calls(lambda: ops.attn_fwd(q, k, v, out=out, balance=False), args.steps, args.warmup)
-        also["c2_flux1024_plain_launch"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        also["c2_flux1024_plain_launch"] = with_rate(time_each(lambda: ops.attn_fwd(q, k, v, out=out, balance=False), n, args.warmup), flops)
         # same shape, BSHD-contiguous memory viewed as BHSD (what a single-GPU Flux block hands over)
         qb, kb, vb = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
         ob = torch.empty(q.shape[0], q.shape[2], q.shape[1], q.shape[3], dtype=q.dtype, device=q.device).transpose(1, 2)
-        _, ms = time_calls(lambda: ops.attn_fwd(qb, kb, vb, out=ob), args.steps, args.warmup)
-        also["c2_flux1024_bshd_view"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        also["c2_flux1024_bshd_view"] = with_rate(time_each(lambda: ops.attn_fwd(qb, kb, vb, out=ob), n, args.warmup), flops)
         # torch's GPU flash attention on the same tensors: what the reference's default backend runs
         try:
-            _, ms = time_calls(lambda: torch_flash(q, k, v), args.steps, args.warmup)
-            also["c2_flux1024_torch_flash_same_gpu"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+            also["c2_flux1024_torch_flash_same_gpu"] = with_rate(time_each(lambda: torch_flash(q, k, v), n, args.warmup), flops)
         except Exception as e:
             also["c2_flux1024_torch_flash_same_gpu"] = {"error": str(e)[:120]}
+        # PixArt-512 self-attention in fp32 (the CPU-runnable configuration), fp32 matrix cores
+        g1 = torch.Generator(device="cpu").manual_seed(1001)
+        q1, k1, v1 = (torch.randn(1, 16, 1024, 72, generator=g1).to(dev) for _ in range(3))
+        f1 = attn_flops(1, 16, 1024, 1024, 72)
+        also["c1_pixart512_fp32"] = with_rate(time_each(lambda: ops.attn_fwd(q1, k1, v1), 50, 10), f1, PEAK_FP32_TFLOPS)
+        del q1, k1, v1
         # ring of 4 KV chunks, merged in fp32 (the cast of the last fold is fused)
         fn = usp._get_attention_function()
-        _, ms = time_calls(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), max(n, args.steps // 4), args.warmup)
-        also["c3_flux_ring4"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        also["c3_flux_ring4"] = with_rate(time_each(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), n, args.warmup), flops)
+        also["host_us_per_call"]["ring4_four_fused_steps"] = host_us_per_call(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), batch=10)
         # the same ring captured once in a HIP graph and replayed (shows whether the eager form is launch-bound)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -254,35 +383,31 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             usp.ring_attn(fn, q, k, v, ring_chunks=4)
-        _, ms = time_calls(graph.replay, max(n, args.steps // 4), args.warmup)
-        also["c3_flux_ring4_graph"] = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1)}
+        also["c3_flux_ring4_graph"] = with_rate(time_each(graph.replay, n, args.warmup), flops)
         del graph
         # the merge kernel alone: bytes per fold = 10*N*D + 12*N
         N = B * H * S
         acc = torch.randn(B, H, S, D, device=dev)
         acc_l = torch.randn(B, H, S, device=dev)
         blk_l = torch.randn(B, H, S, device=dev)
-        _, ms = time_calls(lambda: ops.lse_merge(acc, acc_l, q, blk_l), max(20, n), 5)
+        st = time_each(lambda: ops.lse_merge(acc, acc_l, q, blk_l), 50, 5)
         mbytes = 10.0 * N * D + 12.0 * N
-        also["lse_merge_fold"] = {"us": round(ms * 1e3, 2), "gbs": round(mbytes / ms / 1e6, 1),
-                                  "frac_hbm_peak": round(mbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": mbytes}
+        also["lse_merge_fold"] = {"us": round(st["ms"] * 1e3, 2), "us_min": round(st["ms_min"] * 1e3, 2), "gbs": round(mbytes / st["ms"] / 1e6, 1),
+                                  "frac_hbm_peak": round(mbytes / st["ms"] / 1e6 / PEAK_HBM_GBS, 4), "bytes": mbytes}
         # the last fold of a two-call ring, with the cast to bf16 fused: 12*N*D + 12*N bytes
         fin = torch.empty_like(q)
-        _, ms = time_calls(lambda: ops.lse_merge(acc, acc_l, q, blk_l, final_out=fin), max(20, n), 5)
+        st = time_each(lambda: ops.lse_merge(acc, acc_l, q, blk_l, final_out=fin), 50, 5)
         fbytes = 12.0 * N * D + 12.0 * N
-        also["lse_merge_fold_with_cast"] = {"us": round(ms * 1e3, 2), "gbs": round(fbytes / ms / 1e6, 1),
-                                            "frac_hbm_peak": round(fbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": fbytes}
+        also["lse_merge_fold_with_cast"] = {"us": round(st["ms"] * 1e3, 2), "us_min": round(st["ms_min"] * 1e3, 2), "gbs": round(fbytes / st["ms"] / 1e6, 1),
+                                            "frac_hbm_peak": round(fbytes / st["ms"] / 1e6 / PEAK_HBM_GBS, 4), "bytes": fbytes}
         del acc, qb, kb, vb, fin
         # HunyuanVideo 720p one-GPU head shard
         Bh, Hh, Sh = 1, 3, 118800 + 256
         qh, kh, vh = make_inputs(Bh, Hh, Sh, D, 1004, dev)
-        _, ms = time_calls(lambda: ops.attn_fwd(qh, kh, vh), 5, 2)
         fl = attn_flops(Bh, Hh, Sh, Sh, D)
-        also["c4_hunyuan720p_shard"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1),
-                                        "frac_bf16_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        also["c4_hunyuan720p_shard"] = with_rate(time_each(lambda: ops.attn_fwd(qh, kh, vh), 5, 2), fl, PEAK_BF16_TFLOPS)
         try:
-            _, ms = time_calls(lambda: torch_flash(qh, kh, vh), 5, 2)
-            also["c4_hunyuan720p_shard_torch_flash_same_gpu"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1)}
+            also["c4_hunyuan720p_shard_torch_flash_same_gpu"] = with_rate(time_each(lambda: torch_flash(qh, kh, vh), 3, 1), fl)
         except Exception as e:
             also["c4_hunyuan720p_shard_torch_flash_same_gpu"] = {"error": str(e)[:120]}
         del qh, kh, vh
@@ -290,12 +415,12 @@ def main():
         Bw, Hw, Sw = 1, 5, 75600
         qw, kw, vw = make_inputs(Bw, Hw, Sw, D, 1005, dev, rmsnorm=False)
         (q8, qd), (k8, kd), (v8, vd) = (ops.fp8_quant(t) for t in (qw, kw, vw))
-        _, ms = time_calls(lambda: ops.attn_fwd(q8, k8, v8, q_descale=qd, k_descale=kd, v_descale=vd), 5, 2)
         fl = attn_flops(Bw, Hw, Sw, Sw, D)
-        also["c5_wan720p_shard_fp8"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1),
-                                        "frac_fp8_peak": round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
-        _, ms = time_calls(lambda: ops.fp8_quant(qw), 10, 2)
-        also["fp8_quant_wan_shard"] = {"us": round(ms * 1e3, 1), "gbs": round(qw.numel() * 5.0 / ms / 1e6, 1)}
+        also["c5_wan720p_shard_fp8"] = with_rate(time_each(lambda: ops.attn_fwd(q8, k8, v8, q_descale=qd, k_descale=kd, v_descale=vd), 5, 2), fl, PEAK_FP8_TFLOPS)
+        st = time_each(lambda: ops.fp8_quant(qw), 20, 3)
+        also["fp8_quant_wan_shard"] = {"us": round(st["ms"] * 1e3, 1), "us_min": round(st["ms_min"] * 1e3, 1),
+                                       "gbs": round(qw.numel() * 5.0 / st["ms"] / 1e6, 1),
+                                       "frac_hbm_peak": round(qw.numel() * 5.0 / st["ms"] / 1e6 / PEAK_HBM_GBS, 4)}
         del qw, kw, vw, q8, k8, v8
         # pre-attention prologue (per-head RMSNorm + rotary embedding + BSHD -> BHSD), bf16:
         # bytes per call = 4*N*D (read + write) + 8*S*D (cos and sin rows, read once)
@@ -306,10 +431,10 @@ def main():
             ang = torch.rand(Sp, D, device=dev)
             cs, sn = ang.cos(), ang.sin()
             yp = torch.empty(Bp, Hp, Sp, D, device=dev, dtype=torch.bfloat16)
-            _, ms = time_calls(lambda: prologue.norm_rope(xp, weight=wp, freqs_cis=(cs, sn), sequence_dim=1, out=yp), 20, 3)
+            st = time_each(lambda: prologue.norm_rope(xp, weight=wp, freqs_cis=(cs, sn), sequence_dim=1, out=yp), 20, 3)
             pbytes = 4.0 * xp.numel() + 8.0 * Sp * D
-            also[name] = {"us": round(ms * 1e3, 2), "gbs": round(pbytes / ms / 1e6, 1),
-                          "frac_hbm_peak": round(pbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": pbytes}
+            also[name] = {"us": round(st["ms"] * 1e3, 2), "us_min": round(st["ms_min"] * 1e3, 2), "gbs": round(pbytes / st["ms"] / 1e6, 1),
+                          "frac_hbm_peak": round(pbytes / st["ms"] / 1e6 / PEAK_HBM_GBS, 4), "bytes": pbytes}
             del xp, yp, ang, cs, sn
         # the whole pre-attention step of a Flux block in one launch: norm + rotary + [text; image]
         # concatenation + BSHD -> BHSD of Q and K, re-layout of V (six jobs); bytes = 4 per element
@@ -319,10 +444,10 @@ def main():
         gains = [torch.ones(D, device=dev).bfloat16() for _ in range(4)]
         ang = torch.rand(S_txt + S_img, D, device=dev)
         cs, sn = ang.cos(), ang.sin()
-        _, ms = time_calls(lambda: prologue.flux_joint_qkv(*proj, H, *gains, (cs, sn)), 20, 3)
+        est = time_each(lambda: prologue.flux_joint_qkv(*proj, H, *gains, (cs, sn)), 30, 5)
+        also["host_us_per_call"]["flux_joint_qkv_six_jobs"] = host_us_per_call(lambda: prologue.flux_joint_qkv(*proj, H, *gains, (cs, sn)), batch=20)
         pbytes = 3 * 4.0 * H * D * (S_txt + S_img) + 2 * 8.0 * (S_txt + S_img) * D
-        # the eager call is bound by the Python work of building six jobs; replaying it from a HIP
-        # graph shows the kernel itself
+        # replaying the call from a HIP graph shows the kernel itself
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -332,10 +457,10 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             held = prologue.flux_joint_qkv(*proj, H, *gains, (cs, sn))
-        _, gms = time_calls(graph.replay, 20, 3)
-        also["prologue_flux_block_qkv"] = {"us_eager_call": round(ms * 1e3, 2), "us": round(gms * 1e3, 2),
-                                           "gbs": round(pbytes / gms / 1e6, 1),
-                                           "frac_hbm_peak": round(pbytes / gms / 1e6 / PEAK_HBM_GBS, 4), "bytes": pbytes}
+        gst = time_each(graph.replay, 30, 5)
+        also["prologue_flux_block_qkv"] = {"us_eager_call": round(est["ms"] * 1e3, 2), "us": round(gst["ms"] * 1e3, 2), "us_min": round(gst["ms_min"] * 1e3, 2),
+                                           "gbs": round(pbytes / gst["ms"] / 1e6, 1),
+                                           "frac_hbm_peak": round(pbytes / gst["ms"] / 1e6 / PEAK_HBM_GBS, 4), "bytes": pbytes}
         del graph, held
         result["also"] = also
 

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define XDIT_ATTN_ABI_VERSION 4
+#define XDIT_ATTN_ABI_VERSION 5
 
 typedef enum {
   XDIT_OK = 0,
@@ -75,10 +75,12 @@ typedef struct {
   int32_t out_dtype;           /* xdit_dtype of out: same as dtype for bf16/fp16/fp32; bf16 or fp16 for fp8 */
   int32_t causal;              /* must be 0 */
   int32_t B, H, D;             /* batch, heads (Hq == Hk), head_dim */
-  int32_t reserved0;
+  int32_t rows_per_workgroup;  /* 0 = chosen by the library; 128, 256 or 384 = that workgroup shape
+                                  (bf16 / fp16 / fp8 kernels; a tuning and testing aid) */
   int64_t Sq, Sk, Sk2;         /* query rows; keys in segment 1; keys in segment 2 (0 = none) */
   float softmax_scale;         /* > 0 */
-  float reserved1;
+  int32_t cu_count;            /* 0 = plan the launch for the compute units of the current device;
+                                  > 0 = for that many (tuning, testing, capacity planning) */
   const void* q;
   const void* k;
   const void* v;

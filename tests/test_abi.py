@@ -73,6 +73,10 @@ def _attn_args(**kw):
     (dict(softmax_scale=float("nan")), _lib.XDIT_ERR_INVALID_ARG, "softmax_scale"),
     (dict(out_dtype=_lib.DTYPE_FP32), _lib.XDIT_ERR_INVALID_ARG, "out_dtype"),
     (dict(v_stride=_lib.Strides(0, 0, 4)), _lib.XDIT_ERR_INVALID_ARG, "stride"),
+    # tile loads form "row * stride" with a 24-bit multiply: S strides from 16 MiB up are refused
+    (dict(k_stride=_lib.Strides(0, 128, 1 << 23)), _lib.XDIT_ERR_INVALID_ARG, "too large"),
+    (dict(rows_per_workgroup=100), _lib.XDIT_ERR_INVALID_ARG, "rows_per_workgroup"),
+    (dict(cu_count=-1), _lib.XDIT_ERR_INVALID_ARG, "cu_count"),
     (dict(Sk2=5), _lib.XDIT_ERR_INVALID_ARG, "k2 is NULL"),
     (dict(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16, D=64), _lib.XDIT_ERR_UNSUPPORTED, "fp8"),
 ])
@@ -189,19 +193,17 @@ def test_workspace_query_needs_no_gpu():
     a = _attn_args(B=1, H=24, Sq=4608, Sk=4608)
     for s in ("q_stride", "k_stride", "v_stride", "out_stride"):
         setattr(a, s, _lib.Strides(24 * 4608 * 128, 4608 * 128, 128))
-    os.environ.pop("XDIT_ATTN_ROWS", None)
     need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
     assert need == 32 * (72 // 9 + 1) * 384 * (128 * 2 + 4)
     a.Sk = 64   # a single KV tile cannot be shared
     assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) == 0
 
 
-def test_workspace_of_claimed_ranges(monkeypatch):
+def test_workspace_of_claimed_ranges():
     """A long share (128 remaining query tiles of 256 KV iterations over 256 workgroups = 128
     iterations each) is cut into ranges of 64 iterations that workgroups claim one after the
     other: 4 (+1) slots per remaining tile, plus 256 bytes for the range counter."""
-    monkeypatch.setenv("XDIT_ATTN_ROWS", "384")
-    a = _attn_args(B=1, H=12, Sq=32 * 384, Sk=256 * 64)
+    a = _attn_args(B=1, H=12, Sq=32 * 384, Sk=256 * 64, rows_per_workgroup=384)
     a.q_stride = a.out_stride = _lib.Strides(12 * 32 * 384 * 128, 32 * 384 * 128, 128)
     a.k_stride = a.v_stride = _lib.Strides(12 * 256 * 64 * 128, 256 * 64 * 128, 128)
     need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
@@ -235,8 +237,8 @@ def test_fused_ring_step_rejects_bad_arguments():
     assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "discard_acc_out" in _lib.last_error()
 
 
-def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128):
-    a = _attn_args(B=B, H=H, Sq=Sq, Sk=Sk, Sk2=Sk2, D=D)
+def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128, rows=0, cus=0):
+    a = _attn_args(B=B, H=H, Sq=Sq, Sk=Sk, Sk2=Sk2, D=D, rows_per_workgroup=rows, cu_count=cus)
     if dtype is not None:
         a.dtype = dtype
         a.out_dtype = _lib.DTYPE_BF16
@@ -250,7 +252,7 @@ def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128):
     return p
 
 
-def test_launch_plan_invariants(monkeypatch):
+def test_launch_plan_invariants():
     """The launch geometry for a few hundred random problems: the ranges partition the KV iterations
     of the shared query tiles exactly, every part of a tile has a workspace slot of its own below
     slots_per_tile, the claimers fit the grid, and the workspace holds all slots (host arithmetic
@@ -260,16 +262,12 @@ def test_launch_plan_invariants(monkeypatch):
     seen_counter = seen_fused = seen_separate = seen_plain = 0
     for trial in range(400):
         rows_env = rng.choice([None, "128", "256", "384"])
-        if rows_env is None:
-            monkeypatch.delenv("XDIT_ATTN_ROWS", raising=False)
-        else:
-            monkeypatch.setenv("XDIT_ATTN_ROWS", rows_env)
         fp8 = rng.random() < 0.25
         B, H = rng.choice([1, 1, 2]), rng.choice([1, 3, 5, 12, 24, 40, 64])
         Sq = rng.choice([rng.randint(1, 4000), rng.randint(4000, 40000), rng.randint(40000, 130000)])
         Sk = rng.choice([rng.randint(1, 600), rng.randint(600, 20000), rng.randint(20000, 130000)])
         Sk2 = rng.choice([0, 0, rng.randint(1, 600)])
-        p = _plan(B, H, Sq, Sk, Sk2, dtype=_lib.DTYPE_FP8_E4M3FN if fp8 else None)
+        p = _plan(B, H, Sq, Sk, Sk2, dtype=_lib.DTYPE_FP8_E4M3FN if fp8 else None, rows=int(rows_env or 0))
         rows, nt = p.rows_per_workgroup, p.kv_iterations
         assert rows in (128, 256, 384) and (rows_env is None or rows == int(rows_env))
         assert p.query_tiles == B * H * -(-Sq // rows) and nt == -(-Sk // 64) + -(-Sk2 // 64)
@@ -301,8 +299,7 @@ def test_launch_plan_invariants(monkeypatch):
     assert seen_counter > 10 and seen_fused > 10 and seen_plain > 10
 
 
-def test_launch_plan_of_the_named_shapes(monkeypatch):
-    monkeypatch.delenv("XDIT_ATTN_ROWS", raising=False)
+def test_launch_plan_of_the_named_shapes():
     flux = _plan(1, 24, 4608, 4608)
     assert (flux.rows_per_workgroup, flux.query_tiles, flux.whole_tiles, flux.ranges, flux.range_len,
             flux.claimers, flux.first_claimer, flux.counter, flux.workgroups) == (384, 288, 256, 256, 9, 256, 0, 0, 256)
@@ -332,3 +329,111 @@ def test_launch_plan_of_the_named_shapes(monkeypatch):
     p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
     a.dtype = a.out_dtype = _lib.DTYPE_FP32
     assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == _lib.XDIT_ERR_UNSUPPORTED
+
+
+WALK_HARNESS = r"""
+// Walks every workgroup of a planned launch with the code the kernels run (attn_walk.h) and
+// checks the coverage: stdin holds one launch per line.
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+#include "attn_walk.h"
+struct Geom { int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers; };
+int main() {
+  Geom g; int nt, workgroups, counter, order; long line = 0;
+  while (scanf("%d %d %d %d %d %d %d %d %d %d %d %d", &g.total_tiles, &g.tiles_per_xcd, &g.split_full, &g.split_units, &g.split_len,
+               &g.split_pmax, &g.split_fuse0, &g.split_claimers, &nt, &workgroups, &counter, &order) == 12) {
+    line++;
+    std::vector<int> cover((size_t)g.total_tiles * nt, 0);
+    const int rem = g.total_tiles - g.split_full;
+    std::vector<int> slot_used((size_t)(g.split_units ? rem * g.split_pmax : 0), 0);
+    std::vector<xdit::WorkgroupWalk> walk(workgroups);
+    std::vector<char> live(workgroups, 0);
+    unsigned ticket = 0;
+    for (int w = 0; w < workgroups; w++) live[w] = walk[w].start(g, nt, w);
+    // order 0: a workgroup runs to its end before the next starts; 1: the reverse; 2: one segment per workgroup in turn
+    bool any = true;
+    auto step = [&](int w) {
+      xdit::Segment s;
+      if (!walk[w].next(g, nt, s)) { live[w] = 0; return; }
+      if (s.tile < 0 || s.tile >= g.total_tiles || s.it0 < 0 || s.it1 > nt || s.it0 >= s.it1) { printf("line %ld: bad segment\n", line); exit(1); }
+      for (int t = s.it0; t < s.it1; t++) cover[(size_t)s.tile * nt + t]++;
+      if (s.slot >= 0) {
+        if (s.tile < g.split_full || s.slot >= (long)slot_used.size()) { printf("line %ld: bad slot\n", line); exit(1); }
+        const int r = s.tile - g.split_full;
+        if (s.slot / g.split_pmax != r || s.slot % g.split_pmax >= xdit::shared_tile_parts(g, nt, r)) { printf("line %ld: slot outside its tile\n", line); exit(1); }
+        slot_used[s.slot]++;
+      } else if (s.it0 != 0 || s.it1 != nt) { printf("line %ld: partial tile without a slot\n", line); exit(1); }
+      if (walk[w].wants_claim(counter != 0)) walk[w].claimed(g, ticket++);
+    };
+    while (any) {
+      any = false;
+      for (int i = 0; i < workgroups; i++) {
+        const int w = order == 1 ? workgroups - 1 - i : i;
+        if (order == 2) { if (live[w]) { step(w); any = true; } }
+        else while (live[w]) step(w);
+      }
+    }
+    for (size_t i = 0; i < cover.size(); i++)
+      if (cover[i] != 1) { printf("line %ld: tile %zu iteration %zu covered %d times\n", line, i / nt, i % nt, cover[i]); return 1; }
+    for (int r = 0; r < (g.split_units ? rem : 0); r++)
+      for (int k = 0; k < g.split_pmax; k++)
+        if (slot_used[(size_t)r * g.split_pmax + k] != (k < xdit::shared_tile_parts(g, nt, r) ? 1 : 0)) { printf("line %ld: slots of tile %d\n", line, r); return 1; }
+  }
+  printf("ok %ld\n", line);
+  // thread -> row map of the merge kernel: every chunk of every row held exactly once, by lanes of one wavefront
+  for (int cpr = 1; cpr <= 80; cpr++) {
+    const xdit::MergeMap m = xdit::merge_map(cpr * 8);
+    const int rows = 1000;
+    std::vector<int> held((size_t)rows * cpr, 0);
+    std::vector<long> wave_of(rows, -1);
+    const long waves = (rows + m.rows_per_wave - 1) / m.rows_per_wave;
+    for (long wv = 0; wv < waves; wv++)
+      for (int lane = 0; lane < 64; lane++) {
+        int64_t row; int c0;
+        if (lane / m.lanes_per_row != (int)((lane * m.inv) >> 16)) { printf("merge map: division cpr %d\n", cpr); return 1; }
+        if (!xdit::merge_thread_row(m, wv, lane, row, c0) || row >= rows) continue;
+        if (wave_of[row] >= 0 && wave_of[row] != wv) { printf("merge map: row %ld in two wavefronts, cpr %d\n", (long)row, cpr); return 1; }
+        wave_of[row] = wv;
+        for (int c = c0; c < cpr; c += m.lanes_per_row) held[(size_t)row * cpr + c]++;
+      }
+    for (size_t i = 0; i < held.size(); i++) if (held[i] != 1) { printf("merge map: cpr %d chunk held %d times\n", cpr, held[i]); return 1; }
+  }
+  printf("merge map ok\n");
+  return 0;
+}
+"""
+
+
+def test_every_tile_and_kv_iteration_is_covered_exactly_once(tmp_path):
+    """Coverage of planned launches, walked on the CPU with the very code the kernels run
+    (csrc/attn_walk.h compiled by g++): for compute-unit counts 1..304 (multiples of 8 or not) and
+    random problems, every (query tile, KV iteration) is processed exactly once, every part of a
+    shared tile lands in a slot of its own among those the fold reads, under three execution
+    orders of the workgroups.  Also the merge kernel's thread -> row map for head_dim 8..640."""
+    import random
+    src = tmp_path / "walk.cpp"
+    src.write_text(WALK_HARNESS)
+    exe = tmp_path / "walk"
+    subprocess.check_call(["g++", "-O1", "-std=c++17", "-I", os.path.join(ROOT, "xdit_amd", "csrc"), str(src), "-o", str(exe)])
+    rng = random.Random(99)
+    lines, balanced, odd_balanced = [], 0, 0
+    cases = [(cus, None) for cus in range(1, 305)] + [(rng.choice([0, 8, 64, 100, 252, 255, 256, 304]), i) for i in range(300)]
+    for cus, extra in cases:
+        fp8 = rng.random() < 0.25
+        rows = rng.choice([0, 128, 256, 384])
+        B, H = rng.choice([1, 2]), rng.choice([1, 3, 5, 12, 24])
+        Sq = rng.choice([rng.randint(1, 3000), rng.randint(3000, 40000), rng.randint(3000, 40000)])
+        Sk = rng.choice([rng.randint(1, 600), rng.randint(3500, 12000), rng.randint(3500, 12000)])
+        Sk2 = rng.choice([0, 0, rng.randint(1, 300)])
+        p = _plan(B, H, Sq, Sk, Sk2, dtype=_lib.DTYPE_FP8_E4M3FN if fp8 else None, rows=rows, cus=cus)
+        fuse0 = p.first_claimer if p.ranges and p.first_claimer + p.claimers <= p.whole_tiles else 0x7fffffff
+        full = p.whole_tiles if p.ranges else 0
+        balanced += p.ranges > 0
+        odd_balanced += p.ranges > 0 and full % 8 != 0
+        for order in (0, 1, 2):
+            lines.append("%d %d %d %d %d %d %d %d %d %d %d %d" % (p.query_tiles, -(-p.query_tiles // 8), full, p.ranges, p.range_len,
+                                                             p.slots_per_tile, fuse0, p.claimers, p.kv_iterations, p.workgroups, p.counter, order))
+    assert balanced > 100 and odd_balanced > 20
+    out = subprocess.run([str(exe)], input="\n".join(lines) + "\n", capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.split("\n")[0] == "ok %d" % len(lines) and "merge map ok" in out.stdout, out.stdout[-400:]

@@ -9,7 +9,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libxdit_amd_attn.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 XDIT_OK = 0
 XDIT_ERR_INVALID_ARG = -1
@@ -32,12 +32,12 @@ class AttnArgs(ctypes.Structure):
         ("B", ctypes.c_int32),
         ("H", ctypes.c_int32),
         ("D", ctypes.c_int32),
-        ("reserved0", ctypes.c_int32),
+        ("rows_per_workgroup", ctypes.c_int32),
         ("Sq", ctypes.c_int64),
         ("Sk", ctypes.c_int64),
         ("Sk2", ctypes.c_int64),
         ("softmax_scale", ctypes.c_float),
-        ("reserved1", ctypes.c_float),
+        ("cu_count", ctypes.c_int32),
         ("q", ctypes.c_void_p),
         ("k", ctypes.c_void_p),
         ("v", ctypes.c_void_p),

@@ -36,8 +36,8 @@ int elem_size(int dtype) {
 }
 
 // Every row of a tensor must start on a 16-byte boundary: base aligned, strides multiples of
-// 16 bytes.  The S stride must also keep 64 rows within a 32-bit byte offset (tile loads use
-// "64-bit uniform base + 32-bit per-lane offset" addressing).
+// 16 bytes.  The S stride must stay below 2^24 bytes: tile loads address a row as "64-bit uniform
+// base + 32-bit per-lane offset" and form the offset with a 24-bit multiply (row < 64).
 int check_tensor(const char* name, const void* p, const xdit_strides& st, int esize, int D) {
   if (p == nullptr) return fail(XDIT_ERR_INVALID_ARG, "%s is NULL", name);
   if (!aligned16(p)) return fail(XDIT_ERR_INVALID_ARG, "%s is not 16-byte aligned", name);
@@ -47,7 +47,7 @@ int check_tensor(const char* name, const void* p, const xdit_strides& st, int es
                 name, (long long)st.b, (long long)st.h, (long long)st.s, (long long)m);
   if (st.s < D) return fail(XDIT_ERR_INVALID_ARG, "%s: S stride %lld is smaller than head_dim %d", name, (long long)st.s, D);
   if (st.b < 0 || st.h < 0) return fail(XDIT_ERR_INVALID_ARG, "%s: negative stride", name);
-  if (st.s * esize >= (int64_t(1) << 25))
+  if (st.s * esize >= (int64_t(1) << 24))
     return fail(XDIT_ERR_INVALID_ARG, "%s: S stride of %lld bytes is too large", name, (long long)(st.s * esize));
   return 0;
 }
@@ -70,13 +70,9 @@ bool mfma16_path(const xdit_attn_args* a) {
 int rows_per_block_16(const xdit_attn_args* a) {
   const int D = kernel_head_dim(a->D);
   if (D == 0) return 128;
-  const char* force = std::getenv("XDIT_ATTN_ROWS");  // "128", "256" or "384": testing aid, read per call
-  if (force != nullptr) {
-    const int r = std::atoi(force);
-    if (r == 128 || r == 256 || r == 384) return r;
-  }
+  if (a->rows_per_workgroup != 0) return a->rows_per_workgroup;  // validated by check_tuning
   const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN;
-  const int cus = xdit::resident_cus();
+  const int cus = xdit::resident_cus(a->cu_count);
   const int64_t bh = (int64_t)a->B * a->H;
   const int64_t nt = (a->Sk + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile + (a->Sk2 + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile;
   static const int kRows[3] = {384, 256, 128};
@@ -109,6 +105,15 @@ int rows_per_block_16(const xdit_attn_args* a) {
     if (i == 0 || cost < best_cost) { best = rows; best_cost = cost; }
   }
   return best;
+}
+
+// The two tuning fields of xdit_attn_args.
+int check_tuning(const xdit_attn_args* a) {
+  const int r = a->rows_per_workgroup;
+  if (r != 0 && r != 128 && r != 256 && r != 384)
+    return fail(XDIT_ERR_INVALID_ARG, "rows_per_workgroup %d must be 0, 128, 256 or 384", r);
+  if (a->cu_count < 0 || a->cu_count > 4096) return fail(XDIT_ERR_INVALID_ARG, "cu_count %d must be between 0 and 4096", a->cu_count);
+  return 0;
 }
 
 // Validates one prologue job and fills the kernel parameters.
@@ -191,6 +196,8 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
     return fail(XDIT_ERR_INVALID_ARG, "softmax_scale must be finite and > 0");
   if (a->D <= 0 || a->D % 8 != 0 || a->D > 256) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d: need a multiple of 8, at most 256", a->D);
 
+  if (int rc0 = check_tuning(a)) return rc0;
+
   int out_dtype = a->out_dtype;
   if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
     if (out_dtype != XDIT_DTYPE_BF16 && out_dtype != XDIT_DTYPE_FP16)
@@ -238,6 +245,7 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   p.B = a->B; p.H = a->H;
   p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.scale = a->softmax_scale;
+  p.cu_count = a->cu_count;
   if (acc != nullptr) {  // folded in the epilogue of whole query tiles: no shared last round
     p.acc_out = acc->acc_out; p.acc_lse = acc->acc_lse;
     p.ao_b = acc->acc_out_stride.b; p.ao_h = acc->acc_out_stride.h; p.ao_s = acc->acc_out_stride.s;
@@ -285,9 +293,11 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
       a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30) ||
       (int64_t)a->B * a->H * ((a->Sq + 31) / 32) > (int64_t(1) << 30))
     return fail(XDIT_ERR_INVALID_ARG, "bad shape");
+  if (int rc0 = check_tuning(a)) return rc0;
   xdit::AttnParams p;
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
+  p.cu_count = a->cu_count;
   if (a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128) return (int64_t)xdit::attn_fwd_fp8_workspace(p, rows_per_block_16(a));
   if (!mfma16_path(a)) return 0;
   return (int64_t)xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows_per_block_16(a));
@@ -304,12 +314,14 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
       a->Sk > (int64_t(1) << 30) || a->Sk2 > (int64_t(1) << 30) ||
       (int64_t)a->B * a->H * ((a->Sq + 31) / 32) > (int64_t(1) << 30))
     return fail(XDIT_ERR_INVALID_ARG, "bad shape");
+  if (int rc0 = check_tuning(a)) return rc0;
   const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128;
   const bool b16 = mfma16_path(a);
   if (!fp8 && !b16) return fail(XDIT_ERR_UNSUPPORTED, "no launch plan for this dtype / head_dim (generic kernel: one workgroup per 64 query rows)");
   xdit::AttnParams p, q;
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
+  p.cu_count = a->cu_count;
   const int rows = rows_per_block_16(a);
   const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q);
   const uint32_t size = out->struct_size;

@@ -457,7 +457,7 @@ __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(
 
 // Workgroups of NW wavefronts resident at once: LDS and registers allow two 4-wavefront
 // workgroups per CU, one otherwise.
-static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 2 : 1); }
+static int resident_workgroups(int NW, int planned_cus) { return resident_cus(planned_cus) * (NW == 4 ? 2 : 1); }
 
 template <typename T, int D, int DC, int NW, bool PAD, bool FUSED>
 static hipError_t launch_kernel(const AttnParams& q, hipStream_t stream) {
@@ -481,7 +481,7 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
   // the ring step folds in the epilogue of whole query tiles: no shared last round
-  bind_workspace(q, p, FUSED ? 0 : plan_split(q, rows, resident_workgroups(NW), D, 2, kClaimsPerWorkgroup), rows, D, 2);
+  bind_workspace(q, p, FUSED ? 0 : plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, kClaimsPerWorkgroup), rows, D, 2);
   if constexpr (!FUSED) {
     if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
   }

@@ -319,7 +319,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 2 : 3) void attn_fwd_fp8_kernel(
 }
 
 // Workgroups of NW wavefronts resident at once (3 wavefronts per SIMD by registers; 2 for NW = 8).
-static int resident_workgroups(int NW) { return resident_cus() * (NW == 4 ? 3 : 1); }
+static int resident_workgroups(int NW, int planned_cus) { return resident_cus(planned_cus) * (NW == 4 ? 3 : 1); }
 
 template <typename TO, int NW>
 static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
@@ -328,7 +328,7 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW), D, 2, 1), rows, D, 2);
+  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1), rows, D, 2);
   if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
   dim3 grid(split_grid(q));
   hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW>), grid, dim3(64 * NW), 0, stream, q);
@@ -347,7 +347,7 @@ static size_t workspace_one(const AttnParams& p, AttnParams* plan) {
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  const size_t need = plan_split(q, rows, resident_workgroups(NW), D, 2, 1);
+  const size_t need = plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1);
   if (plan != nullptr) *plan = q;
   return need;
 }

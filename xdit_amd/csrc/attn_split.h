@@ -9,74 +9,34 @@
 
 namespace xdit {
 
-// Workgroup -> segments of work.  `seg(tile, it0, it1, part_out, part_lse)` processes KV tiles
-// [it0, it1) of query tile `tile`; part_out == nullptr means "write the final result".
-// Plain launch (split_units == 0): workgroup = one query tile over all KV tiles.  Balanced launch:
-// the first split_full workgroups each take a whole query tile; the KV iterations of the
-// remaining query tiles, laid end to end, are cut into split_units ranges of split_len
-// iterations.  A range may cover the end of one query tile and the start of the next.  The
-// ranges are processed by split_claimers workgroups: the workgroups split_fuse0 .. split_full-1
-// (the last to be dispatched) after their own query tile, so that no compute unit waits for a
-// new workgroup to be dispatched in between, or, with fewer whole tiles than that
-// (split_fuse0 > split_full), workgroups of their own, split_full .. split_full+claimers-1.
-// Claimer c starts with range c; when there are more ranges than claimers (split_counter !=
-// nullptr) every further range is taken from a counter in device memory, so that compute units
-// that run faster (the clocks of the eight XCDs differ by several per cent) take more of them.
-// TO is the output element type, ROWS the query rows per workgroup.
+// Runs the segments of this workgroup (see WorkgroupWalk in attn_walk.h for who does what).
+// `seg(tile, it0, it1, part_out, part_lse)` processes KV tiles [it0, it1) of query tile `tile`;
+// part_out == nullptr means "write the final result", otherwise the normalised partial result and
+// its log-sum-exp go to that workspace slot.  TO is the output element type, ROWS the query rows
+// per workgroup.
 template <typename TO, int ROWS, int D, typename Seg>
 __device__ __forceinline__ void run_workgroup(const AttnParams& p, Seg seg) {
   const int nt = (p.Sk + kKeysPerTile - 1) / kKeysPerTile + (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-  __shared__ int next_unit;
-  const int w = blockIdx.x;
-  // What this workgroup does: a whole query tile first (whole_tile >= 0), then ranges (claimer).
-  int whole_tile = -1;
-  int u_next = -1;  // the range to start with, < 0: none
-  if (p.split_units == 0) {
-    whole_tile = xcd_tile_index(w, p.tiles_per_xcd);
-    if (whole_tile >= p.total_tiles) return;
-  } else if (w < p.split_full) {
-    whole_tile = xcd_tile_index(w, p.split_full >> 3);
-    u_next = w - p.split_fuse0;
-  } else {
-    u_next = w - p.split_full;
-  }
-  const int rem_iters = (p.total_tiles - p.split_full) * nt;
-  int u = 0, lin = 0, lin_end = 0;
+  __shared__ unsigned ticket;
+  WorkgroupWalk walk;
+  if (!walk.start(p, nt, (int)blockIdx.x)) return;
   bool first = true;
-  for (;;) {  // one segment per turn; a single call site keeps one copy of the kernel body
-    int tile, it0, it1;
+  Segment s;
+  while (walk.next(p, nt, s)) {  // one segment per turn; a single call site keeps one copy of the kernel body
     TO* part_out = nullptr;
     float* part_lse = nullptr;
-    if (whole_tile >= 0) {
-      tile = whole_tile; it0 = 0; it1 = nt;
-      whole_tile = -1;
-    } else {
-      if (lin >= lin_end) {  // the next range
-        if (u_next < 0 || u_next >= p.split_units) return;
-        u = u_next;
-        u_next = -1;
-        lin = u * p.split_len;
-        lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
-      }
-      const int r = lin / nt;               // which of the remaining query tiles
-      it0 = lin - r * nt;
-      it1 = (lin_end - r * nt) < nt ? (lin_end - r * nt) : nt;
-      const int part = u - (r * nt) / p.split_len;  // ranges are consecutive: index within the tile
-      const int64_t slot = (int64_t)r * p.split_pmax + part;
-      tile = p.split_full + r;
-      part_out = (TO*)p.ws_out + slot * ROWS * D;
-      part_lse = p.ws_lse + slot * ROWS;
-      lin += it1 - it0;
+    if (s.slot >= 0) {
+      part_out = (TO*)p.ws_out + s.slot * ROWS * D;
+      part_lse = p.ws_lse + s.slot * ROWS;
     }
     if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
-    seg(tile, it0, it1, part_out, part_lse);
+    seg(s.tile, s.it0, s.it1, part_out, part_lse);
     first = false;
-    if (whole_tile < 0 && lin >= lin_end && u_next < 0 && p.split_counter != nullptr && p.split_units != 0 &&
-        (w >= p.split_fuse0 || w >= p.split_full)) {
-      __syncthreads();  // everyone has read next_unit of the previous claim
-      if (threadIdx.x == 0) next_unit = p.split_claimers + (int)atomicAdd(p.split_counter, 1u);
+    if (walk.wants_claim(p.split_counter != nullptr)) {
+      __syncthreads();  // everyone has read the ticket of the previous claim
+      if (threadIdx.x == 0) ticket = atomicAdd(p.split_counter, 1u);
       __syncthreads();
-      u_next = next_unit;
+      walk.claimed(p, ticket);
     }
   }
 }
@@ -107,9 +67,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, c
   const int h = bh - b * p.H;
   const int qrow = qt * rows_per_block + row;
   if (qrow >= p.Sq) return;
-  const int first_unit = (r * nt) / p.split_len;
-  const int last_unit = ((r + 1) * nt - 1) / p.split_len;
-  const int nparts = last_unit - first_unit + 1;
+  const int nparts = shared_tile_parts(p, nt, r);
   const float* lsep = p.ws_lse + ((int64_t)r * p.split_pmax) * rows_per_block + row;
   typedef __attribute__((ext_vector_type(8))) T vec8;
   const T* part0 = (const T*)p.ws_out + (((int64_t)r * p.split_pmax) * rows_per_block + row) * D + col;
@@ -160,8 +118,10 @@ static inline int current_device_slot() {
   return dev % kMaxDevices;
 }
 
-// Compute units of the current device (cached; concurrent first calls store the same value).
-static inline int resident_cus() {
+// Compute units of the current device (cached; concurrent first calls store the same value), or
+// the number the caller plans for.
+static inline int resident_cus(int planned = 0) {
+  if (planned > 0) return planned;
   static std::atomic<int> cus[kMaxDevices];
   const int slot = current_device_slot();
   int n = cus[slot].load(std::memory_order_relaxed);

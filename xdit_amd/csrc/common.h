@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "attn_walk.h"
+
 namespace xdit {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -51,6 +53,7 @@ struct AttnParams {
   int tiles_per_xcd;  // ceil(total_tiles / 8)
   float scale;        // softmax scale
   int d_actual;       // head_dim of the tensors when the kernel is built for a larger one (0: the kernel's own)
+  int cu_count;       // compute units the launch is planned for (0: those of the current device)
   // balanced launch (see attn_fwd_16_kernel); all zero for a plain launch
   int split_full;     // query tiles handled whole, by the first workgroups
   int split_units;    // workgroups sharing the KV iterations of the remaining query tiles
@@ -100,13 +103,5 @@ __device__ __forceinline__ float fold_value(float acc, float blk, float w) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
-
-// Workgroup index -> work tile, XCD-aware.  Workgroups are handed to the 8 XCDs round-robin
-// (workgroup i runs on XCD i % 8).  Giving XCD x the contiguous tile range
-// [x * tiles_per_xcd, (x+1) * tiles_per_xcd) keeps the query tiles of one (batch, head) — which
-// all stream the same K/V — on one XCD, so that K/V is fetched into that XCD's L2 once.
-__device__ __forceinline__ int xcd_tile_index(int block, int tiles_per_xcd) {
-  return (block & 7) * tiles_per_xcd + (block >> 3);
-}
 
 }  // namespace xdit

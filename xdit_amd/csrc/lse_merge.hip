@@ -11,10 +11,14 @@
 // _attention.py:161-163), and `final_out`, when given, receives the merged rows in the block
 // dtype (the epilogue cast at ring_flash_attn.py:145) in the same pass.
 //
-// Memory-bound: every thread moves 8 consecutive head_dim elements (32 B of fp32 accumulator,
-// 16 B of 16-bit block) per row; a row's D/8 threads are adjacent lanes, so accumulator accesses
-// coalesce to full rows.  The lse values of a row are loaded by each of its threads (served by
-// one L1 line) and stored by the first.
+// Memory-bound: a thread moves 8 consecutive head_dim elements (32 B of fp32 accumulator, 16 B
+// of 16-bit block) at a time; the D/8 chunks of a row are held by adjacent lanes of ONE
+// wavefront (MergeMap in attn_walk.h), so accumulator accesses coalesce to full rows and a
+// wavefront covers whole rows only.  Every lane of a row reads the row's accumulated
+// log-sum-exp before the row's first lane overwrites it in place; with the row inside one
+// wavefront, program order guarantees that for every head_dim (rows that straddled two
+// wavefronts, as they would at head_dim 72 with a flat thread -> chunk map, could see the new
+// value in the later wavefront).
 #include "common.h"
 #include "launchers.h"
 
@@ -57,12 +61,11 @@ template <> struct Load8<_Float16> {
 };
 
 template <typename TB, typename TF, bool HAS_FINAL>
-__global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p) {
-  const int tpr = p.D >> 3;  // threads per row
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t row = gid / tpr;
-  const int col = (int)(gid - row * tpr) * 8;
-  if (row >= p.rows) return;
+__global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p, const MergeMap map) {
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  int64_t row;
+  int chunk0;
+  if (!merge_thread_row(map, wave, threadIdx.x & 63, row, chunk0) || row >= p.rows) return;
   // row -> (b, h, s); consecutive rows walk s fastest, then h, then b
   const int s = (int)(row % p.S);
   const int64_t bh = row / p.S;
@@ -71,45 +74,51 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p) {
 
   const float* bl = p.block_lse + b * p.bl_b + h * p.bl_h + s * p.bl_s;
   float* al = p.acc_lse + b * p.al_b + h * p.al_h + s * p.al_s;
-  float* ao = p.acc_out + b * p.ao_b + h * p.ao_h + s * p.ao_s + col;
-  const TB* bo = (const TB*)p.block_out + b * p.bo_b + h * p.bo_h + s * p.bo_s + col;
+  float* ao_row = p.acc_out + b * p.ao_b + h * p.ao_h + s * p.ao_s;
+  const TB* bo_row = (const TB*)p.block_out + b * p.bo_b + h * p.bo_h + s * p.bo_s;
 
-  float xb[8], xo[8];
-  Load8<TB>::ld(bo, xb);
   const float blse = *bl;
-  float new_lse;
-  if (p.first) {
-#pragma unroll
-    for (int i = 0; i < 8; i++) xo[i] = xb[i];
-    new_lse = blse;
-  } else {
-    Load8<float>::ld(ao, xo);
-    const float lse = *al;
-    const float w = sigmoid(blse - lse);
-#pragma unroll
-    for (int i = 0; i < 8; i++) xo[i] = fold_value(xo[i], xb[i], w);
+  float w = 0.f, new_lse = blse;
+  if (!p.first) {
+    const float lse = *al;  // read by every lane of the row before its first lane stores below
+    w = sigmoid(blse - lse);
     new_lse = lse - log_sigmoid(lse - blse);
   }
-  Load8<float>::st(ao, xo);
-  if (col == 0) *al = new_lse;
-  if (HAS_FINAL) {
-    TF* fo = (TF*)p.final_out + b * p.fo_b + h * p.fo_h + s * p.fo_s + col;
-    Load8<TF>::st(fo, xo);
+  for (int chunk = chunk0; chunk < map.cpr; chunk += map.lanes_per_row) {  // one turn unless head_dim > 512
+    const int col = chunk * 8;
+    float xb[8], xo[8];
+    Load8<TB>::ld(bo_row + col, xb);
+    if (p.first) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) xo[i] = xb[i];
+    } else {
+      Load8<float>::ld(ao_row + col, xo);
+#pragma unroll
+      for (int i = 0; i < 8; i++) xo[i] = fold_value(xo[i], xb[i], w);
+    }
+    Load8<float>::st(ao_row + col, xo);
+    if (HAS_FINAL) {
+      TF* fo = (TF*)p.final_out + b * p.fo_b + h * p.fo_h + s * p.fo_s + col;
+      Load8<TF>::st(fo, xo);
+    }
   }
+  if (chunk0 == 0) *al = new_lse;
 }
 
 template <typename TB>
 static hipError_t launch_tb(const MergeParams& p, int final_dtype, hipStream_t stream) {
-  const int64_t threads = p.rows * (p.D >> 3);
-  dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+  const MergeMap map = merge_map(p.D);
+  const int64_t waves = (p.rows + map.rows_per_wave - 1) / map.rows_per_wave;
+  if ((waves + 3) / 4 > 0x7fffffffLL) return hipErrorInvalidValue;
+  dim3 grid((unsigned)((waves + 3) / 4)), block(256);
   if (p.final_out == nullptr) {
-    hipLaunchKernelGGL((lse_merge_kernel<TB, float, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((lse_merge_kernel<TB, float, false>), grid, block, 0, stream, p, map);
   } else if (final_dtype == 0) {
-    hipLaunchKernelGGL((lse_merge_kernel<TB, __bf16, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((lse_merge_kernel<TB, __bf16, true>), grid, block, 0, stream, p, map);
   } else if (final_dtype == 1) {
-    hipLaunchKernelGGL((lse_merge_kernel<TB, _Float16, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((lse_merge_kernel<TB, _Float16, true>), grid, block, 0, stream, p, map);
   } else {
-    hipLaunchKernelGGL((lse_merge_kernel<TB, float, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((lse_merge_kernel<TB, float, true>), grid, block, 0, stream, p, map);
   }
   return hipGetLastError();
 }

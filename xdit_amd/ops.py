@@ -41,16 +41,33 @@ def _check4(name, t, device):
 
 
 def _stream(device):
-    return torch.cuda.current_stream(device).cuda_stream
+    return torch._C._cuda_getCurrentRawStream(device.index if device.index is not None else torch.cuda.current_device())
+
+
+class _on_device:
+    """`with torch.cuda.device(device)` only when the device is not the current one already."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, device):
+        idx = device.index
+        self.ctx = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
 
 
 _WORKSPACE = {}
 
 
-def _workspace(device, nbytes):
+def _workspace(device, stream, nbytes):
     """Per-device scratch tensor for balanced launches, grown on demand.  Calls on one stream are
     ordered, so one buffer per (device, stream) can be reused from call to call."""
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    key = (device, stream)
     buf = _WORKSPACE.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
@@ -58,18 +75,26 @@ def _workspace(device, nbytes):
     return buf
 
 
-def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
-             q_descale=None, k_descale=None, v_descale=None, out_dtype=None, out=None,
-             return_lse=True, balance=True, _acc=None):
-    """Non-causal attention forward on logical BHSD tensors -> (out BHSD, lse (B,H,Sq) fp32).
+# Launch tuning passed to the library with every attention call (fields of xdit_attn_args):
+# rows_per_workgroup 0 = the library's choice, else 128 / 256 / 384; cu_count 0 = the device's
+# compute units, else plan the launch as for that many.  Tests and sweeps set these.
+TUNING = {"rows_per_workgroup": 0, "cu_count": 0}
 
-    `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
-    with `k`/`v`.  For fp8 (torch.float8_e4m3fn) inputs the descales are (B, H) fp32 tensors.
-    `balance=False` withholds the scratch buffer with which the library evens out the last round
-    of workgroups (results then come from one workgroup per query tile).
-    """
-    if (k2 is None) != (v2 is None):
-        raise ValueError("k2 and v2 should be None or not None simultaneously.")
+# Argument structs are filled once per call signature (shapes, strides, dtypes, options) and kept:
+# a later call with the same signature only patches the pointers and the stream.
+_PLANS = {}
+_PLANS_MAX = 512
+
+
+class _AttnPlan:
+    __slots__ = ("args", "need", "shape", "out_dtype", "ring")
+
+
+def _sig(t):
+    return None if t is None else (t.shape, t.stride(), t.device)
+
+
+def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype, out, lse, acc):
     device = q.device
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check4(name, t, device)
@@ -78,69 +103,143 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
         raise ValueError("q %s, k %s, v %s do not agree (Hq must equal Hk)" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise ValueError("q, k, v must share a dtype")
-    Sk = k.shape[2]
-    Sk2 = 0
+    a = _lib.AttnArgs()
+    a.struct_size = ctypes.sizeof(_lib.AttnArgs)
+    a.dtype = _code(q.dtype)
+    a.out_dtype = _code(out_dtype)
+    a.causal = 1 if causal else 0
+    a.B, a.H, a.D = B, H, D
+    a.rows_per_workgroup = int(TUNING["rows_per_workgroup"])
+    a.cu_count = int(TUNING["cu_count"])
+    a.Sq, a.Sk = Sq, k.shape[2]
+    a.softmax_scale = float(softmax_scale)
+    a.q_stride, a.k_stride, a.v_stride = _strides(q), _strides(k), _strides(v)
     if k2 is not None:
         _check4("k2", k2, device)
         _check4("v2", v2, device)
         if k2.shape[0] != B or k2.shape[1] != H or k2.shape[3] != D or v2.shape != k2.shape or k2.dtype != q.dtype or v2.dtype != q.dtype:
             raise ValueError("joint k2/v2 do not match q/k/v")
-        Sk2 = k2.shape[2]
-    dt = _code(q.dtype)
-    if out_dtype is None:
-        out_dtype = torch.bfloat16 if q.dtype == torch.float8_e4m3fn else q.dtype
-    if softmax_scale is None:
-        softmax_scale = float(D) ** -0.5
-    if out is None:
-        if _acc is None:
-            out = torch.empty((B, H, Sq, D), dtype=out_dtype, device=device)
-    else:
+        if k2.shape[2] > 0:
+            a.Sk2 = k2.shape[2]
+            a.k2_stride, a.v2_stride = _strides(k2), _strides(v2)
+    if out is not None:
         _check4("out", out, device)
         if tuple(out.shape) != (B, H, Sq, D) or out.dtype != out_dtype:
             raise ValueError("out has the wrong shape or dtype")
-    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=device) if return_lse else None
-
-    a = _lib.AttnArgs()
-    a.struct_size = ctypes.sizeof(_lib.AttnArgs)
-    a.dtype = dt
-    a.out_dtype = _code(out_dtype)
-    a.causal = 1 if causal else 0
-    a.B, a.H, a.D = B, H, D
-    a.Sq, a.Sk, a.Sk2 = Sq, Sk, Sk2
-    a.softmax_scale = float(softmax_scale)
-    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
-    a.q_stride, a.k_stride, a.v_stride = _strides(q), _strides(k), _strides(v)
-    if k2 is not None and Sk2 > 0:
-        a.k2, a.v2 = k2.data_ptr(), v2.data_ptr()
-        a.k2_stride, a.v2_stride = _strides(k2), _strides(v2)
-    if out is not None:
-        a.out = out.data_ptr()
         a.out_stride = _strides(out)
+    else:
+        a.out_stride = _lib.Strides(H * Sq * D, Sq * D, D)  # a new BHSD-contiguous tensor per call
     if lse is not None:
-        a.lse = lse.data_ptr()
+        if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, Sq) or lse.device != device or (Sq > 1 and lse.stride(2) != 1):
+            raise ValueError("lse must be a (B, H, Sq) fp32 tensor on %s with a unit stride over Sq" % (device,))
         a.lse_stride_b, a.lse_stride_h = lse.stride(0), lse.stride(1)
-    keep = []
-    for name, d in (("q_descale", q_descale), ("k_descale", k_descale), ("v_descale", v_descale)):
+    else:
+        a.lse_stride_b, a.lse_stride_h = H * Sq, Sq
+    for name, d in zip(("q_descale", "k_descale", "v_descale"), descales):
         if d is None:
             continue
         if q.dtype != torch.float8_e4m3fn:
             raise ValueError("%s is only meaningful for fp8 inputs" % name)
         if d.dtype != torch.float32 or tuple(d.shape) != (B, H) or d.device != device:
             raise ValueError("%s must be a (B, H) fp32 tensor on %s" % (name, device))
-        d = d.contiguous()
-        keep.append(d)
-        setattr(a, name, d.data_ptr())
-        a.descale_stride_b, a.descale_stride_h = d.stride(0), d.stride(1)
-    a.stream = _stream(device)
-    with torch.cuda.device(device):
+        a.descale_stride_b, a.descale_stride_h = H, 1  # descales are passed contiguous
+    plan = _AttnPlan()
+    plan.args = a
+    plan.shape = (B, H, Sq, D)
+    plan.out_dtype = out_dtype
+    plan.ring = None
+    plan.need = 0
+    if acc is not None:
+        acc_out, acc_lse, first, discard = acc
+        _check4("acc_out", acc_out, device)
+        if acc_out.dtype != torch.float32 or acc_lse.dtype != torch.float32:
+            raise ValueError("acc_out and acc_lse must be fp32")
+        if tuple(acc_out.shape) != (B, H, Sq, D) or tuple(acc_lse.shape) != (B, H, Sq) or acc_lse.device != device:
+            raise ValueError("accumulator shape mismatch")
+        r = _lib.RingAcc()
+        r.struct_size = ctypes.sizeof(_lib.RingAcc)
+        r.first = 1 if first else 0
+        r.discard_acc_out = 1 if discard else 0
+        r.acc_out_stride = _strides(acc_out)
+        r.acc_lse_stride = _lib.Strides(acc_lse.stride(0), acc_lse.stride(1), acc_lse.stride(2))
+        plan.ring = r
+    else:
+        with _on_device(device):
+            need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
+        if need < 0:
+            _lib.check(need)
+        plan.need = need
+    return plan
+
+
+def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
+             q_descale=None, k_descale=None, v_descale=None, out_dtype=None, out=None,
+             return_lse=True, balance=True, lse=None, _acc=None):
+    """Non-causal attention forward on logical BHSD tensors -> (out BHSD, lse (B,H,Sq) fp32).
+
+    `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
+    with `k`/`v`.  For fp8 (torch.float8_e4m3fn) inputs the descales are (B, H) fp32 tensors.
+    `out` / `lse` receive the results when given (new tensors otherwise).
+    `balance=False` withholds the scratch buffer with which the library evens out the last round
+    of workgroups (results then come from one workgroup per query tile).
+    """
+    if (k2 is None) != (v2 is None):
+        raise ValueError("k2 and v2 should be None or not None simultaneously.")
+    if not isinstance(q, torch.Tensor) or q.ndim != 4:
+        raise ValueError("q must be a 4-D tensor (B, H, S, D)")
+    device = q.device
+    if out_dtype is None:
+        out_dtype = torch.bfloat16 if q.dtype == torch.float8_e4m3fn else q.dtype
+    if softmax_scale is None:
+        softmax_scale = float(q.shape[-1]) ** -0.5
+    if lse is not None:
+        return_lse = True
+    acc_sig = None if _acc is None else (_sig(_acc[0]), _sig(_acc[1]), _acc[2], _acc[3])
+    key = (q.dtype, out_dtype, device, _sig(q), _sig(k), _sig(v), _sig(k2), _sig(v2), _sig(out), _sig(lse),
+           k.dtype, v.dtype, float(softmax_scale), bool(causal), q_descale is not None, k_descale is not None,
+           v_descale is not None, acc_sig, TUNING["rows_per_workgroup"], TUNING["cu_count"])
+    plan = _PLANS.get(key)
+    if plan is None:
+        plan = _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, (q_descale, k_descale, v_descale),
+                                out_dtype, out, lse, _acc)
+        if len(_PLANS) >= _PLANS_MAX:
+            _PLANS.clear()
+        _PLANS[key] = plan
+    else:
+        for d in (q_descale, k_descale, v_descale):  # values the signature does not cover
+            if d is not None and (d.dtype != torch.float32 or tuple(d.shape) != plan.shape[:2] or d.device != device):
+                raise ValueError("descales must be (B, H) fp32 tensors on %s" % (device,))
+    if out is None and _acc is None:
+        out = torch.empty(plan.shape, dtype=out_dtype, device=device)
+    if lse is None and return_lse and _acc is None:
+        lse = torch.empty(plan.shape[:3], dtype=torch.float32, device=device)
+    a = plan.args
+    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    if a.Sk2:
+        a.k2, a.v2 = k2.data_ptr(), v2.data_ptr()
+    a.out = out.data_ptr() if out is not None else None
+    a.lse = lse.data_ptr() if lse is not None else None
+    keep = None
+    if q_descale is not None or k_descale is not None or v_descale is not None:
+        keep = [None if d is None else d.contiguous() for d in (q_descale, k_descale, v_descale)]
+        a.q_descale, a.k_descale, a.v_descale = (None if d is None else d.data_ptr() for d in keep)
+    stream = _stream(device)
+    a.stream = stream
+    L = _lib.lib()
+    with _on_device(device):
         if _acc is not None:
-            _lib.check(_lib.lib().xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(_acc)))
-            return out, lse
-        need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) if balance else 0
-        if need > 0:
-            ws = _workspace(device, need)
-            a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
-        _lib.check(_lib.lib().xdit_attn_fwd(ctypes.byref(a)))
+            r = plan.ring
+            r.acc_out, r.acc_lse = _acc[0].data_ptr(), _acc[1].data_ptr()
+            rc = L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r))
+        else:
+            if balance and plan.need > 0:
+                ws = _workspace(device, stream, plan.need)
+                a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+            else:
+                a.workspace, a.workspace_bytes = None, 0
+            rc = L.xdit_attn_fwd(ctypes.byref(a))
+    if rc != 0:
+        _lib.check(rc)
     return out, lse
 
 
@@ -156,6 +255,8 @@ def launch_plan(q, k, k2=None):
     a.B, a.H, a.Sq, a.D = q.shape
     a.Sk = k.shape[2]
     a.Sk2 = 0 if k2 is None else k2.shape[2]
+    a.rows_per_workgroup = int(TUNING["rows_per_workgroup"])
+    a.cu_count = int(TUNING["cu_count"])
     p = _lib.LaunchPlan()
     p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
     _lib.check(_lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)))
@@ -174,23 +275,10 @@ def attn_fwd_accumulate(q, k, v, acc_out, acc_lse, first=False, final_out=None, 
     followed by `lse_merge` would, without the block ever reaching memory.  `first` initialises
     the accumulator; `final_out` (logical BHSD, q's dtype) also receives the merged rows;
     `discard_acc_out` skips the write-back of acc_out (last step).  Returns (acc_out, acc_lse)."""
-    device = q.device
-    _check4("acc_out", acc_out, device)
-    B, H, Sq, D = q.shape
-    if acc_out.dtype != torch.float32 or acc_lse.dtype != torch.float32:
-        raise ValueError("acc_out and acc_lse must be fp32")
-    if tuple(acc_out.shape) != (B, H, Sq, D) or tuple(acc_lse.shape) != (B, H, Sq) or acc_lse.device != device:
-        raise ValueError("accumulator shape mismatch")
     if discard_acc_out and final_out is None:
         raise ValueError("discard_acc_out needs final_out")
-    r = _lib.RingAcc()
-    r.struct_size = ctypes.sizeof(_lib.RingAcc)
-    r.first = 1 if first else 0
-    r.discard_acc_out = 1 if discard_acc_out else 0
-    r.acc_out, r.acc_lse = acc_out.data_ptr(), acc_lse.data_ptr()
-    r.acc_out_stride = _strides(acc_out)
-    r.acc_lse_stride = _lib.Strides(acc_lse.stride(0), acc_lse.stride(1), acc_lse.stride(2))
-    attn_fwd(q, k, v, softmax_scale=softmax_scale, k2=k2, v2=v2, out=final_out, return_lse=False, _acc=r)
+    attn_fwd(q, k, v, softmax_scale=softmax_scale, k2=k2, v2=v2, out=final_out, return_lse=False,
+             _acc=(acc_out, acc_lse, bool(first), bool(discard_acc_out)))
     return acc_out, acc_lse
 
 
@@ -225,7 +313,7 @@ def lse_merge(acc_out, acc_lse, block_out, block_lse, first=False, final_out=Non
         a.final_dtype = _code(final_out.dtype)
         a.final_out_stride = _strides(final_out)
     a.stream = _stream(device)
-    with torch.cuda.device(device):
+    with _on_device(device):
         _lib.check(_lib.lib().xdit_lse_merge(ctypes.byref(a)))
     return acc_out, acc_lse
 
@@ -252,7 +340,7 @@ def fp8_quant(x, per_tensor=False, scale=None, hadamard_block=0):
         a.scale_in = scale.data_ptr()
     a.x_stride, a.y_stride = _strides(x), _strides(y)
     a.stream = _stream(device)
-    with torch.cuda.device(device):
+    with _on_device(device):
         _lib.check(_lib.lib().xdit_fp8_quant(ctypes.byref(a)))
     return y, descale
 
@@ -325,7 +413,7 @@ def qk_prologue(x, weight=None, eps=1e-6, norm=None, rotary_emb=None, rope="inte
     """
     keep = []
     a, out = _prologue_job(x, weight, eps, norm, rotary_emb, rope, rope_row0, rope_rows, out, keep)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _lib.check(_lib.lib().xdit_qk_prologue(ctypes.byref(a)))
     return out
 
@@ -342,6 +430,6 @@ def qk_prologue_batch(jobs):
                                j.get("rope", "interleaved"), j.get("rope_row0", 0), j.get("rope_rows"), j.get("out"), keep)
         arr[i] = a
         outs.append(out)
-    with torch.cuda.device(jobs[0]["x"].device):
+    with _on_device(jobs[0]["x"].device):
         _lib.check(_lib.lib().xdit_qk_prologue_batch(arr, len(jobs)))
     return outs
