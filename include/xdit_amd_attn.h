@@ -114,6 +114,22 @@ int xdit_attn_fwd(const xdit_attn_args* args);
 int64_t xdit_attn_workspace_bytes(const xdit_attn_args* args);
 
 /*
+ * xdit_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same arguments, results and kernels, but
+ * the scratch of the balanced launch is a fixed array of XDIT_ATTN_NOALLOC_SCRATCH_BYTES inside
+ * the library (one copy per GPU, held until the process ends) instead of a workspace of the
+ * caller; args->workspace is ignored.  Nothing is allocated or freed by the call.  A problem whose
+ * xdit_attn_workspace_bytes exceeds the array is rejected with XDIT_ERR_INVALID_ARG (use
+ * xdit_attn_fwd with a workspace then); Flux-1024 (B=1, H=24, S=4608, D=128) needs 28.75 MB.
+ * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (two streams,
+ * two threads) race on it and must be serialised by the caller; calls on one stream are ordered.
+ * The array needs no clearing between calls (the range counter in it is reset by a kernel of each
+ * call).  No counterpart in the reference.
+ */
+#define XDIT_ATTN_NOALLOC_SCRATCH_BYTES (32 * 1024 * 1024)
+int xdit_attn_fwd_noalloc(const xdit_attn_args* args);
+
+/*
  * How xdit_attn_fwd would launch this problem when given the workspace it asks for (pointers of
  * `args` are not inspected): for tests, tuning and capacity planning.  The query rows are cut
  * into `query_tiles` tiles of `rows_per_workgroup` rows, each with `kv_iterations` tiles of 64

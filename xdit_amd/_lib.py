@@ -169,7 +169,7 @@ class PrologueArgs(ctypes.Structure):
 NORM_NONE, NORM_HEAD, NORM_TOKEN = 0, 1, 2
 ROPE_NONE, ROPE_INTERLEAVED, ROPE_SPLIT_HALF, ROPE_WAN = 0, 1, 2, 3
 
-EXPORTS = ("xdit_attn_fwd", "xdit_attn_fwd_accumulate", "xdit_attn_workspace_bytes", "xdit_attn_launch_plan", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_qk_prologue_batch", "xdit_attn_last_error", "xdit_attn_abi_version")
+EXPORTS = ("xdit_attn_fwd", "xdit_attn_fwd_noalloc", "xdit_attn_fwd_accumulate", "xdit_attn_workspace_bytes", "xdit_attn_launch_plan", "xdit_lse_merge", "xdit_fp8_quant", "xdit_qk_prologue", "xdit_qk_prologue_batch", "xdit_attn_last_error", "xdit_attn_abi_version")
 
 _lib = None
 _lock = threading.Lock()
@@ -191,6 +191,8 @@ def lib():
         L = ctypes.CDLL(LIB_PATH)
         L.xdit_attn_fwd.argtypes = [ctypes.POINTER(AttnArgs)]
         L.xdit_attn_fwd.restype = ctypes.c_int
+        L.xdit_attn_fwd_noalloc.argtypes = [ctypes.POINTER(AttnArgs)]
+        L.xdit_attn_fwd_noalloc.restype = ctypes.c_int
         L.xdit_attn_fwd_accumulate.argtypes = [ctypes.POINTER(AttnArgs), ctypes.POINTER(RingAcc)]
         L.xdit_attn_fwd_accumulate.restype = ctypes.c_int
         L.xdit_attn_launch_plan.argtypes = [ctypes.POINTER(AttnArgs), ctypes.POINTER(LaunchPlan)]

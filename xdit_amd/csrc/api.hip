@@ -11,6 +11,12 @@
 #include "attn_split.h"
 #include "launchers.h"
 
+// Scratch of xdit_attn_fwd_noalloc: the balanced launch's partial results and range counter live
+// here instead of in a caller workspace.  One copy per GPU the library runs on, held until the
+// process ends.  In host code the array's name is only a handle for hipGetSymbolAddress; the
+// device address it yields (per device) is what the launches receive.
+static __device__ __align__(256) unsigned char scratch[XDIT_ATTN_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -275,6 +281,35 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
 }
 
 int xdit_attn_fwd(const xdit_attn_args* a) { return attn_fwd_impl(a, nullptr); }
+
+int xdit_attn_fwd_noalloc(const xdit_attn_args* a) {
+  g_err[0] = 0;
+  if (a == nullptr) return fail(XDIT_ERR_INVALID_ARG, "args is NULL");
+  const int64_t need = xdit_attn_workspace_bytes(a);  // validates struct_size, shape and tuning fields
+  if (need < 0) return (int)need;
+  if (need > (int64_t)XDIT_ATTN_NOALLOC_SCRATCH_BYTES)
+    return fail(XDIT_ERR_INVALID_ARG,
+                "this problem needs %lld bytes of scratch, xdit_attn_fwd_noalloc holds %lld: call xdit_attn_fwd with a workspace of the caller",
+                (long long)need, (long long)XDIT_ATTN_NOALLOC_SCRATCH_BYTES);
+  xdit_attn_args b = *a;
+  b.workspace = nullptr;
+  b.workspace_bytes = 0;
+  if (need > 0) {
+    // device address of this GPU's copy of the array, looked up once per device with that device current
+    static std::atomic<void*> scratch_ptr[xdit::kMaxDevices];
+    const int slot = xdit::current_device_slot();
+    void* ptr = scratch_ptr[slot].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+      const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || ptr == nullptr)
+        return fail(XDIT_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+      scratch_ptr[slot].store(ptr, std::memory_order_release);
+    }
+    b.workspace = ptr;
+    b.workspace_bytes = (int64_t)XDIT_ATTN_NOALLOC_SCRATCH_BYTES;
+  }
+  return attn_fwd_impl(&b, nullptr);
+}
 
 int xdit_attn_fwd_accumulate(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   if (acc == nullptr) {

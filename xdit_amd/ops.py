@@ -174,7 +174,7 @@ def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype
 
 def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
              q_descale=None, k_descale=None, v_descale=None, out_dtype=None, out=None,
-             return_lse=True, balance=True, lse=None, _acc=None):
+             return_lse=True, balance=True, lse=None, noalloc=False, _acc=None):
     """Non-causal attention forward on logical BHSD tensors -> (out BHSD, lse (B,H,Sq) fp32).
 
     `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
@@ -182,6 +182,9 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     `out` / `lse` receive the results when given (new tensors otherwise).
     `balance=False` withholds the scratch buffer with which the library evens out the last round
     of workgroups (results then come from one workgroup per query tile).
+    `noalloc=True` goes through the library's entry point that allocates nothing: the scratch is
+    a fixed buffer inside the library (problems that need more than it holds raise ValueError),
+    and `out` (and `lse` when `return_lse`) must be given.
     """
     if (k2 is None) != (v2 is None):
         raise ValueError("k2 and v2 should be None or not None simultaneously.")
@@ -192,6 +195,8 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
         out_dtype = torch.bfloat16 if q.dtype == torch.float8_e4m3fn else q.dtype
     if softmax_scale is None:
         softmax_scale = float(q.shape[-1]) ** -0.5
+    if noalloc and (out is None or (return_lse and lse is None) or _acc is not None):
+        raise ValueError("noalloc needs out (and lse) from the caller and is not available for the ring step")
     if lse is not None:
         return_lse = True
     acc_sig = None if _acc is None else (_sig(_acc[0]), _sig(_acc[1]), _acc[2], _acc[3])
@@ -231,6 +236,9 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
             r = plan.ring
             r.acc_out, r.acc_lse = _acc[0].data_ptr(), _acc[1].data_ptr()
             rc = L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r))
+        elif noalloc:
+            a.workspace, a.workspace_bytes = None, 0
+            rc = L.xdit_attn_fwd_noalloc(ctypes.byref(a))
         else:
             if balance and plan.need > 0:
                 ws = _workspace(device, stream, plan.need)
