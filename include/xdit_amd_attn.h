@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define XDIT_ATTN_ABI_VERSION 5
+#define XDIT_ATTN_ABI_VERSION 6
 
 typedef enum {
   XDIT_OK = 0,
@@ -81,6 +81,16 @@ typedef struct {
   float softmax_scale;         /* > 0 */
   int32_t cu_count;            /* 0 = plan the launch for the compute units of the current device;
                                   > 0 = for that many (tuning, testing, capacity planning) */
+  int32_t deterministic;       /* != 0: results reproducible bit for bit from call to call.  0 (the
+                                  value the reference passes for its `deterministic` option at every
+                                  call site): a balanced launch may hand KV iterations of a shared
+                                  query tile to whichever workgroup is free, so results are
+                                  reproducible only to rounding (the last bit of some outputs) */
+  int32_t workspace_preserved; /* != 0: the caller vouches that nothing but this library has written
+                                  `workspace` since an earlier call of this library that was given the
+                                  same pointer (with 0 here on the first call after allocating it):
+                                  the counters the library keeps at its start are then still zero, and
+                                  a small initialisation launch per call is spared.  0 is always valid */
   const void* q;
   const void* k;
   const void* v;
@@ -108,8 +118,9 @@ int xdit_attn_fwd(const xdit_attn_args* args);
  * (out, lse) pairs go through the workspace and are folded by a second small kernel.
  * Returns 0 when nothing would be gained, a negative xdit_status for invalid arguments
  * (pointers are not inspected).  Passing no or too small a workspace to xdit_attn_fwd is always
- * valid: the launch is then simply not balanced.  The workspace contents are undefined after the
- * call and need no initialisation.  No counterpart in the reference (its kernels are vendor code).
+ * valid: the launch is then simply not balanced.  The workspace needs no initialisation and may
+ * be used for anything else between calls (see workspace_preserved for what a caller gains by
+ * leaving it alone).  No counterpart in the reference (its kernels are vendor code).
  */
 int64_t xdit_attn_workspace_bytes(const xdit_attn_args* args);
 
@@ -156,6 +167,11 @@ typedef struct {
   int32_t first_claimer;
   int32_t counter;
   int32_t workgroups;          /* grid of the attention kernel */
+  int32_t streamed;            /* != 0: streamed sharing instead of ranges: the `claimers` workgroups are dealt
+                                  out over the shared tiles in contiguous groups; every member owns
+                                  `range_len` KV iterations of its tile and draws the others one at a
+                                  time from the tile's counter (not with deterministic != 0) */
+  int32_t reserved0;
 } xdit_launch_plan;
 
 int xdit_attn_launch_plan(const xdit_attn_args* args, xdit_launch_plan* plan);

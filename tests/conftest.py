@@ -18,3 +18,14 @@ def gpu():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(params=["deterministic", "streamed"])
+def sharing_mode(request, monkeypatch):
+    """Runs a GPU test twice: with the `deterministic` option of the attention call (fixed work
+    geometry, bit-reproducible results) and with the library's default, under which the KV
+    iterations of shared query tiles may go to whichever workgroup is free (results reproducible
+    to rounding)."""
+    from xdit_amd import ops
+    monkeypatch.setitem(ops.TUNING, "deterministic", 1 if request.param == "deterministic" else 0)
+    return request.param

@@ -194,7 +194,10 @@ def test_workspace_query_needs_no_gpu():
     for s in ("q_stride", "k_stride", "v_stride", "out_stride"):
         setattr(a, s, _lib.Strides(24 * 4608 * 128, 4608 * 128, 128))
     need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
-    assert need == 32 * (72 // 9 + 1) * 384 * (128 * 2 + 4)
+    # streamed sharing: 8 workgroups per shared tile, one partial result each, plus the tiles' counters
+    assert need == 16384 + 32 * 8 * 384 * (128 * 2 + 4)   # 16 KiB of counters lead every workspace
+    a.deterministic = 1   # fixed ranges of 9 KV iterations: up to 72 / 9 + 1 parts per tile
+    assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) == 16384 + 32 * (72 // 9 + 1) * 384 * (128 * 2 + 4)
     a.Sk = 64   # a single KV tile cannot be shared
     assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) == 0
 
@@ -202,13 +205,13 @@ def test_workspace_query_needs_no_gpu():
 def test_workspace_of_claimed_ranges():
     """A long share (128 remaining query tiles of 256 KV iterations over 256 workgroups = 128
     iterations each) is cut into ranges of 64 iterations that workgroups claim one after the
-    other: 4 (+1) slots per remaining tile, plus 256 bytes for the range counter."""
+    other: 4 (+1) slots per remaining tile, behind the 16 KiB of counters that lead a workspace."""
     a = _attn_args(B=1, H=12, Sq=32 * 384, Sk=256 * 64, rows_per_workgroup=384)
     a.q_stride = a.out_stride = _lib.Strides(12 * 32 * 384 * 128, 32 * 384 * 128, 128)
     a.k_stride = a.v_stride = _lib.Strides(12 * 256 * 64 * 128, 256 * 64 * 128, 128)
     need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
     parts = 128 * (256 // 64 + 1) * 384 * (128 * 2 + 4)
-    assert parts % 256 == 0 and need == parts + 256
+    assert need == 16384 + parts
 
 
 def test_fused_ring_step_rejects_bad_arguments():
@@ -237,8 +240,8 @@ def test_fused_ring_step_rejects_bad_arguments():
     assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "discard_acc_out" in _lib.last_error()
 
 
-def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128, rows=0, cus=0):
-    a = _attn_args(B=B, H=H, Sq=Sq, Sk=Sk, Sk2=Sk2, D=D, rows_per_workgroup=rows, cu_count=cus)
+def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128, rows=0, cus=0, det=True):
+    a = _attn_args(B=B, H=H, Sq=Sq, Sk=Sk, Sk2=Sk2, D=D, rows_per_workgroup=rows, cu_count=cus, deterministic=1 if det else 0)
     if dtype is not None:
         a.dtype = dtype
         a.out_dtype = _lib.DTYPE_BF16
@@ -295,7 +298,7 @@ def test_launch_plan_invariants():
             last = ((r + 1) * nt - 1) // p.range_len
             assert last < p.ranges and last - first + 1 <= p.slots_per_tile
         parts = rem * p.slots_per_tile * rows * (128 * 2 + 4)
-        assert p.workspace_bytes == (((parts + 255) & ~255) + 256 if p.counter else parts)
+        assert p.workspace_bytes == 16384 + parts
     assert seen_counter > 10 and seen_fused > 10 and seen_plain > 10
 
 
@@ -303,6 +306,10 @@ def test_launch_plan_of_the_named_shapes():
     flux = _plan(1, 24, 4608, 4608)
     assert (flux.rows_per_workgroup, flux.query_tiles, flux.whole_tiles, flux.ranges, flux.range_len,
             flux.claimers, flux.first_claimer, flux.counter, flux.workgroups) == (384, 288, 256, 256, 9, 256, 0, 0, 256)
+    fs = _plan(1, 24, 4608, 4608, det=False)   # the default: streamed sharing, 8 members per shared tile owning 2 iterations each
+    assert (fs.rows_per_workgroup, fs.whole_tiles, fs.ranges, fs.range_len, fs.claimers, fs.first_claimer, fs.counter, fs.workgroups,
+            fs.streamed, fs.slots_per_tile) == (384, 256, 256, 2, 256, 0, 1, 256, 1, 8)
+    assert _plan(1, 3, 118800 + 256, 118800 + 256, det=False).streamed == 0   # long shares keep their claimed ranges
     hv = _plan(1, 3, 118800 + 256, 118800 + 256)
     assert (hv.rows_per_workgroup, hv.query_tiles, hv.whole_tiles, hv.kv_iterations) == (384, 933, 768, 1861)
     assert (hv.ranges, hv.range_len, hv.claimers, hv.first_claimer, hv.counter, hv.workgroups) == (1536, 200, 256, 512, 1, 768)
@@ -338,12 +345,13 @@ WALK_HARNESS = r"""
 #include <cstdlib>
 #include <vector>
 #include "attn_walk.h"
-struct Geom { int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers; };
+struct Geom { int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers, split_dyn, split_s0; };
 int main() {
   Geom g; int nt, workgroups, counter, order; long line = 0;
-  while (scanf("%d %d %d %d %d %d %d %d %d %d %d %d", &g.total_tiles, &g.tiles_per_xcd, &g.split_full, &g.split_units, &g.split_len,
-               &g.split_pmax, &g.split_fuse0, &g.split_claimers, &nt, &workgroups, &counter, &order) == 12) {
+  while (scanf("%d %d %d %d %d %d %d %d %d %d %d %d %d %d", &g.total_tiles, &g.tiles_per_xcd, &g.split_full, &g.split_units, &g.split_len,
+               &g.split_pmax, &g.split_fuse0, &g.split_claimers, &nt, &workgroups, &counter, &order, &g.split_dyn, &g.split_s0) == 14) {
     line++;
+    std::vector<unsigned> tile_counter(g.total_tiles, 0u);
     std::vector<int> cover((size_t)g.total_tiles * nt, 0);
     const int rem = g.total_tiles - g.split_full;
     std::vector<int> slot_used((size_t)(g.split_units ? rem * g.split_pmax : 0), 0);
@@ -358,13 +366,22 @@ int main() {
       if (!walk[w].next(g, nt, s)) { live[w] = 0; return; }
       if (s.tile < 0 || s.tile >= g.total_tiles || s.it0 < 0 || s.it1 > nt || s.it0 >= s.it1) { printf("line %ld: bad segment\n", line); exit(1); }
       for (int t = s.it0; t < s.it1; t++) cover[(size_t)s.tile * nt + t]++;
+      if (s.dyn >= 0) {  // streamed sharing: draw the tile's other iterations one at a time, as the kernel does
+        if (s.tile != g.split_full + s.dyn || s.pool0 < s.it1 || !g.split_dyn) { printf("line %ld: bad streamed segment\n", line); exit(1); }
+        // order 2 interleaves the draws of the group's members; the others let one member take the whole pool
+        for (int n = 0; order != 2 || n < 3; n++) {
+          const unsigned tk = tile_counter[s.dyn]++;
+          if ((int)tk >= nt - s.pool0) break;
+          cover[(size_t)s.tile * nt + s.pool0 + tk]++;
+        }
+      }
       if (s.slot >= 0) {
         if (s.tile < g.split_full || s.slot >= (long)slot_used.size()) { printf("line %ld: bad slot\n", line); exit(1); }
         const int r = s.tile - g.split_full;
         if (s.slot / g.split_pmax != r || s.slot % g.split_pmax >= xdit::shared_tile_parts(g, nt, r)) { printf("line %ld: slot outside its tile\n", line); exit(1); }
         slot_used[s.slot]++;
       } else if (s.it0 != 0 || s.it1 != nt) { printf("line %ld: partial tile without a slot\n", line); exit(1); }
-      if (walk[w].wants_claim(counter != 0)) walk[w].claimed(g, ticket++);
+      if (walk[w].wants_claim(counter != 0 && !g.split_dyn)) walk[w].claimed(g, ticket++);
     };
     while (any) {
       any = false;
@@ -374,6 +391,11 @@ int main() {
         else while (live[w]) step(w);
       }
     }
+    if (g.split_dyn)  // whoever comes last drains what is left of every pool (the kernel's members draw until the pool is empty)
+      for (int r = 0; r < rem; r++) {
+        const int pool0 = xdit::shared_tile_parts(g, nt, r) * g.split_s0;
+        for (;;) { const unsigned tk = tile_counter[r]++; if ((int)tk >= nt - pool0) break; cover[(size_t)(g.split_full + r) * nt + pool0 + tk]++; }
+      }
     for (size_t i = 0; i < cover.size(); i++)
       if (cover[i] != 1) { printf("line %ld: tile %zu iteration %zu covered %d times\n", line, i / nt, i % nt, cover[i]); return 1; }
     for (int r = 0; r < (g.split_units ? rem : 0); r++)
@@ -417,7 +439,7 @@ def test_every_tile_and_kv_iteration_is_covered_exactly_once(tmp_path):
     exe = tmp_path / "walk"
     subprocess.check_call(["g++", "-O1", "-std=c++17", "-I", os.path.join(ROOT, "xdit_amd", "csrc"), str(src), "-o", str(exe)])
     rng = random.Random(99)
-    lines, balanced, odd_balanced = [], 0, 0
+    lines, balanced, odd_balanced, streamed = [], 0, 0, 0
     cases = [(cus, None) for cus in range(1, 305)] + [(rng.choice([0, 8, 64, 100, 252, 255, 256, 304]), i) for i in range(300)]
     for cus, extra in cases:
         fp8 = rng.random() < 0.25
@@ -426,14 +448,16 @@ def test_every_tile_and_kv_iteration_is_covered_exactly_once(tmp_path):
         Sq = rng.choice([rng.randint(1, 3000), rng.randint(3000, 40000), rng.randint(3000, 40000)])
         Sk = rng.choice([rng.randint(1, 600), rng.randint(3500, 12000), rng.randint(3500, 12000)])
         Sk2 = rng.choice([0, 0, rng.randint(1, 300)])
-        p = _plan(B, H, Sq, Sk, Sk2, dtype=_lib.DTYPE_FP8_E4M3FN if fp8 else None, rows=rows, cus=cus)
+        p = _plan(B, H, Sq, Sk, Sk2, dtype=_lib.DTYPE_FP8_E4M3FN if fp8 else None, rows=rows, cus=cus, det=rng.random() < 0.3)
+        streamed += p.streamed
         fuse0 = p.first_claimer if p.ranges and p.first_claimer + p.claimers <= p.whole_tiles else 0x7fffffff
         full = p.whole_tiles if p.ranges else 0
         balanced += p.ranges > 0
         odd_balanced += p.ranges > 0 and full % 8 != 0
         for order in (0, 1, 2):
-            lines.append("%d %d %d %d %d %d %d %d %d %d %d %d" % (p.query_tiles, -(-p.query_tiles // 8), full, p.ranges, p.range_len,
-                                                             p.slots_per_tile, fuse0, p.claimers, p.kv_iterations, p.workgroups, p.counter, order))
-    assert balanced > 100 and odd_balanced > 20
+            lines.append("%d %d %d %d %d %d %d %d %d %d %d %d %d %d" % (p.query_tiles, -(-p.query_tiles // 8), full, p.ranges, p.range_len,
+                                                                   p.slots_per_tile, fuse0, p.claimers, p.kv_iterations, p.workgroups, p.counter, order,
+                                                                   p.streamed, p.range_len if p.streamed else 0))
+    assert balanced > 100 and odd_balanced > 20 and streamed > 20
     out = subprocess.run([str(exe)], input="\n".join(lines) + "\n", capture_output=True, text=True)
     assert out.returncode == 0 and out.stdout.split("\n")[0] == "ok %d" % len(lines) and "merge map ok" in out.stdout, out.stdout[-400:]

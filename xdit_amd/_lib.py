@@ -9,7 +9,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libxdit_amd_attn.so")
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 XDIT_OK = 0
 XDIT_ERR_INVALID_ARG = -1
@@ -38,6 +38,8 @@ class AttnArgs(ctypes.Structure):
         ("Sk2", ctypes.c_int64),
         ("softmax_scale", ctypes.c_float),
         ("cu_count", ctypes.c_int32),
+        ("deterministic", ctypes.c_int32),
+        ("workspace_preserved", ctypes.c_int32),
         ("q", ctypes.c_void_p),
         ("k", ctypes.c_void_p),
         ("v", ctypes.c_void_p),
@@ -104,6 +106,8 @@ class LaunchPlan(ctypes.Structure):
         ("first_claimer", ctypes.c_int32),
         ("counter", ctypes.c_int32),
         ("workgroups", ctypes.c_int32),
+        ("streamed", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
     ]
 
 

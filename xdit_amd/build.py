@@ -14,6 +14,8 @@ OBJDIR = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libxdit_amd_attn.so")
 SOURCES = ["api.hip", "attn_fwd_16.hip", "attn_fwd_16_ring.hip", "attn_fwd_fp8.hip", "attn_fwd_f32.hip", "lse_merge.hip", "fp8_quant.hip", "qk_prologue.hip"]
 FLAGS = [
+    # an atomic under a one-lane branch stays one plain atomic whose result is awaited where it is used
+    "-mllvm", "-amdgpu-atomic-optimizer-strategy=None",
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed-fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -99,7 +99,8 @@ int rows_per_block_16(const xdit_attn_args* a) {
     xdit::AttnParams q;
     std::memset(&q, 0, sizeof(q));
     q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
-    xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup);
+    q.deterministic = a->deterministic;
+    xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8);
     // every segment costs a few iterations' worth of prologue and epilogue (about 13 us: 5
     // iterations at head_dim 128, 9 at head_dim 64), the combine pass about as much again
     const double ovh = D == 64 ? 9.0 : 5.0;
@@ -252,6 +253,7 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.scale = a->softmax_scale;
   p.cu_count = a->cu_count;
+  p.deterministic = a->deterministic;
   if (acc != nullptr) {  // folded in the epilogue of whole query tiles: no shared last round
     p.acc_out = acc->acc_out; p.acc_lse = acc->acc_lse;
     p.ao_b = acc->acc_out_stride.b; p.ao_h = acc->acc_out_stride.h; p.ao_s = acc->acc_out_stride.s;
@@ -260,6 +262,7 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
     p.acc_store = acc->discard_acc_out == 0;
   } else if (a->workspace != nullptr && a->workspace_bytes > 0 && aligned16(a->workspace)) {
     p.ws_out = a->workspace;
+    p.ws_preserved = a->workspace_preserved != 0;
     p.ws_bytes = (size_t)a->workspace_bytes;
   }
   hipStream_t stream = (hipStream_t)a->stream;
@@ -294,6 +297,7 @@ int xdit_attn_fwd_noalloc(const xdit_attn_args* a) {
   xdit_attn_args b = *a;
   b.workspace = nullptr;
   b.workspace_bytes = 0;
+  b.workspace_preserved = 0;
   if (need > 0) {
     // device address of this GPU's copy of the array, looked up once per device with that device current
     static std::atomic<void*> scratch_ptr[xdit::kMaxDevices];
@@ -307,6 +311,7 @@ int xdit_attn_fwd_noalloc(const xdit_attn_args* a) {
     }
     b.workspace = ptr;
     b.workspace_bytes = (int64_t)XDIT_ATTN_NOALLOC_SCRATCH_BYTES;
+    b.workspace_preserved = 1;  // the array starts out zeroed and only this library writes it
   }
   return attn_fwd_impl(&b, nullptr);
 }
@@ -333,6 +338,7 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.cu_count = a->cu_count;
+  p.deterministic = a->deterministic;
   if (a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128) return (int64_t)xdit::attn_fwd_fp8_workspace(p, rows_per_block_16(a));
   if (!mfma16_path(a)) return 0;
   return (int64_t)xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows_per_block_16(a));
@@ -357,6 +363,7 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.cu_count = a->cu_count;
+  p.deterministic = a->deterministic;
   const int rows = rows_per_block_16(a);
   const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q);
   const uint32_t size = out->struct_size;
@@ -372,7 +379,9 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
   out->slots_per_tile = q.split_pmax;
   out->claimers = q.split_claimers;
   out->first_claimer = q.split_units ? (q.split_fuse0 <= q.split_full ? q.split_fuse0 : q.split_full) : 0;
-  out->counter = q.split_units > q.split_claimers ? 1 : 0;
+  out->counter = xdit::split_counters(q) > 0 ? 1 : 0;
+  out->streamed = q.split_dyn;
+  if (q.split_dyn) out->range_len = q.split_s0;
   out->workgroups = (int32_t)xdit::split_grid(q);
   return XDIT_OK;
 }

@@ -13,7 +13,7 @@ static size_t workspace_one(const AttnParams& p, AttnParams* plan) {
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  const size_t need = plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, kClaimsPerWorkgroup);
+  const size_t need = plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, kClaimsPerWorkgroup, true);
   if (plan != nullptr) *plan = q;
   return need;
 }

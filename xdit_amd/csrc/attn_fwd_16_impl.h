@@ -28,6 +28,13 @@
 #include "attn_split.h"
 #include "launchers.h"
 
+// Timestamp hooks of an instrumented build: a translation unit that defines XDIT_TRACE_POINT(part, k)
+// before including this file records when a workgroup passes point k (0 entry of a segment,
+// 1 first K/V tile landed, 2 end of the KV loop, 3 end of the epilogue); nothing otherwise.
+#ifndef XDIT_TRACE_POINT
+#define XDIT_TRACE_POINT(part, k)
+#endif
+
 namespace xdit {
 
 constexpr int kRowsPerWave = 32;
@@ -39,19 +46,63 @@ constexpr int kPrefetch = 4;
 constexpr int kStagePitchBytes = 64 * 2 + 8;
 constexpr int kStageBytesPerWave = kRowsPerWave * kStagePitchBytes + kRowsPerWave * 4;  // + one fp32 per row (ring step)
 
-// One segment of work: the query tile `tile`, KV tiles [it0, it1).  With `part_out == nullptr` the
-// normalised result goes to the output tensors; otherwise the segment is one PART of a query tile
-// whose KV range is shared between workgroups, and its normalised partial output (in T) and
-// log-sum-exp go to the workspace slot (part_out, part_lse), [row][D] and [row], to be folded by
-// attn_combine_kernel.
+// LDS of a workgroup: the first K/V buffer, then a region that holds the second K/V buffer during
+// the KV loop and the output staging blocks of the wavefronts in the epilogue.  The epilogue thus
+// leaves the first buffer alone, and the first K/V tile of the workgroup's next segment is loaded
+// into it while the rows of the current one are stored.
+template <int D, int NW>
+constexpr int lds_bytes_16() {
+  return TileGeom<D>::BUF_BYTES + (TileGeom<D>::BUF_BYTES > NW * kStageBytesPerWave ? TileGeom<D>::BUF_BYTES : NW * kStageBytesPerWave);
+}
+
+// The work of one workgroup: its segments (WorkgroupWalk), one after the other.  A segment is the
+// query tile `tile` and KV tiles [it0, it1), plus, under streamed sharing, further KV tiles of the
+// same query tile drawn one at a time from the tile's counter.  With slot < 0 the normalised
+// result goes to the output tensors; otherwise the segment is one PART of a query tile whose KV
+// range is shared between workgroups, and its normalised partial output (in T) and log-sum-exp
+// go to the workspace slot, [row][D] and [row], to be folded by attn_combine_kernel.
+// Between two segments the Q fragments and the first K/V tile of the next one are requested
+// before the rows of the current one are stored, so their latency hides behind the epilogue.
 // PAD: the tensors' head_dim (p.d_actual, a multiple of 8) is smaller than D; the missing columns
-// are zeros in the Q fragments and in LDS (cleared here, never written by the tile loads) and are
+// are zeros in the Q fragments and in LDS (cleared once, never written by the tile loads) and are
 // not stored.  DC (a multiple of 16, d_actual <= DC <= D) is the head_dim the two products are
 // computed over: LDS tiles keep the geometry of D, contraction steps (of 16) and output blocks
 // (of 32) past DC are left out.
+// The lane's index within its wavefront, computed where it is called (two instructions) instead
+// of being kept in a register through the KV loop; not merged with other calls by the compiler.
+__device__ __forceinline__ int lane_now() {
+  int x;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(x));
+  return x;
+}
+
+// One ticket from a counter in device memory (device-scope atomic add of 1, relaxed), for a branch
+// that a single lane takes.  The operands are formed right here rather than kept in registers
+// through the KV loop around it.
+__device__ __forceinline__ unsigned draw_ticket(unsigned* counter) {
+  unsigned one = 1;
+  asm volatile("" : "+v"(one));
+  return __hip_atomic_fetch_add(counter, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The launch geometry the walker reads, gathered from the kernel arguments when needed.
+struct WalkGeom {
+  int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers, split_dyn, split_s0;
+};
+typedef const __attribute__((address_space(4))) AttnParams* ParamsPtr;
+__device__ __forceinline__ WalkGeom walk_geom(ParamsPtr pp) {
+  WalkGeom g = {pp->total_tiles, pp->tiles_per_xcd, pp->split_full, pp->split_units, pp->split_len, pp->split_pmax,
+                pp->split_fuse0, pp->split_claimers, pp->split_dyn, pp->split_s0};
+  return g;
+}
+
+// The kernel's only argument is read in place, through a pointer to the kernel-argument segment
+// that is made opaque to the compiler after every KV loop: what a segment's prologue and
+// epilogue need is then loaded (scalar loads) when it is needed instead of being kept in
+// registers across the loop, which leaves the loop the registers.
 template <typename T, int D, int DC, int NW, bool PAD, bool FUSED>
-__device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char* smem, const int tile,
-                                             const int it0, const int it1, T* part_out, float* part_lse) {
+__device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
+  ParamsPtr pp = (ParamsPtr)__builtin_amdgcn_kernarg_segment_ptr();
   constexpr int kWaves = NW;
   constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
   typedef typename Mfma16<T>::vec8 vec8;
@@ -63,396 +114,474 @@ __device__ __forceinline__ void attn_segment(const AttnParams& p, unsigned char*
   constexpr int kStagePitch = kStagePitchBytes;   // LDS row pitch of the output staging block
   constexpr int kStageBytes = kStageBytesPerWave;
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nt1 = (pp->Sk + kKeysPerTile - 1) / kKeysPerTile;
+  const int nt = nt1 + (pp->Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  __shared__ unsigned ticket;   // range claims
+  __shared__ int drawn[2];      // streamed sharing: KV tile of the stream position after next, by parity
+  WorkgroupWalk walk;
+  Segment seg;
+  {
+    const WalkGeom g = walk_geom(pp);
+    if (!walk.start(g, nt, (int)blockIdx.x) || !walk.next(g, nt, seg)) return;
+  }
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int dact = PAD ? pp->d_actual : D;
+  const int lane = lane_now();   // for the set-up below; later code asks again
   const int l32 = lane & 31;
   const int hh = lane >> 5;
-
-  const int bh = tile / p.nq_tiles;
-  const int qt = tile - bh * p.nq_tiles;
-  const int b = bh / p.H;
-  const int h = bh - b * p.H;
-
-  // ---- Q fragments: B operand of S^T, lane = (query l32, contraction half hh) -------------
-  const int qrow = qt * kRowsPerBlock + wave * kRowsPerWave + l32;
-  const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
-  const T* qptr = (const T*)p.q + b * p.qs_b + h * p.qs_h + (int64_t)qrow_c * p.qs_s + hh * 8;
-  const int dact = PAD ? p.d_actual : D;
-  vec8 qf[KSTEPS];
-#pragma unroll
-  for (int ks = 0; ks < KSTEPS; ks++) {
-    if (!PAD || ks * 16 + hh * 8 < dact) {
-      qf[ks] = *(const vec8*)(qptr + ks * 16);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; e++) qf[ks][e] = (T)0.f;
-    }
-  }
 
   // ---- direct global->LDS tile loads ------------------------------------------------------
   // A tile is 2*NG pieces of 1 KiB (K pieces 0..NG-1, then V pieces): piece g of K (or V) holds
   // rows g, g+NG, g+2NG, ...; wavefront w loads pieces w, w+NW, w+2NW, ...; within a piece
   // lane -> (slot = lane / lanes-per-row, 16-byte column = lane % lanes-per-row).  A load is
   // "uniform 64-bit tile base + per-lane 32-bit byte offset".
-  const T* kbase1 = (const T*)p.k + b * p.ks_b + h * p.ks_h;
-  const T* vbase1 = (const T*)p.v + b * p.vs_b + h * p.vs_h;
-  const T* kbase2 = p.Sk2 > 0 ? (const T*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
-  const T* vbase2 = p.Sk2 > 0 ? (const T*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
   constexpr int LANES_PER_ROW = G::ROW_BYTES / 16;
   // Loader wavefronts: the first LW wavefronts each load PAIRS (K piece g, V piece g) pairs,
   // g = wave + LW * i, with one row index per lane for both pieces of a pair.
   constexpr int LW = kWaves < 8 ? kWaves : 8;
   constexpr int PAIRS = G::NG / LW;
   static_assert(G::NG % LW == 0, "pieces must divide evenly over the loader wavefronts");
-  const int ld_row0 = G::NG * (lane / LANES_PER_ROW) + wave;  // row of this lane in pair 0
-  const unsigned ld_colb = (lane % LANES_PER_ROW) * 16;       // byte offset inside the row
-  const bool ld_on = !PAD || ld_colb < (unsigned)dact * 2;    // lanes of columns the tensors do not have stay idle
+  int ld_row0 = G::NG * (lane / LANES_PER_ROW) + wave;   // row of this lane in pair 0
+  unsigned ld_colb = (lane % LANES_PER_ROW) * 16;        // byte offset inside the row
+  asm volatile("" : "+v"(ld_row0), "+v"(ld_colb));       // kept as two registers through the KV loop
+  const bool ld_on = !PAD || ld_colb < (unsigned)dact * 2;  // lanes of columns the tensors do not have stay idle
   const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS unsigned char*)smem;
   const unsigned ld_kdst = lds_base + wave * G::K_PITCH;      // LDS address of K piece `wave`, buffer 0
   const unsigned ld_vdst = lds_base + G::K_BYTES + wave * G::V_PITCH;
 
-  const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
-  const int nt2 = (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-  const int nt = nt1 + nt2;
-
-  // Stream position: base pointers of the next tile to load, byte strides, keys left in its segment.
-  const T* ld_kp;
-  const T* ld_vp;
-  unsigned ld_kss, ld_vss;
-  int64_t ld_kstep, ld_vstep;
-  int ld_left;
-  auto seek_tile = [&](int t) {
-    if (t < nt1) {
-      ld_kp = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
-      ld_vp = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
-      ld_kss = (unsigned)(p.ks_s * 2); ld_vss = (unsigned)(p.vs_s * 2);
-      ld_kstep = kKeysPerTile * p.ks_s; ld_vstep = kKeysPerTile * p.vs_s;
-      ld_left = p.Sk - t * kKeysPerTile;
-    } else {
-      ld_kp = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
-      ld_vp = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
-      ld_kss = (unsigned)(p.k2s_s * 2); ld_vss = (unsigned)(p.v2s_s * 2);
-      ld_kstep = kKeysPerTile * p.k2s_s; ld_vstep = kKeysPerTile * p.v2s_s;
-      ld_left = p.Sk2 - (t - nt1) * kKeysPerTile;
-    }
-  };
-  // Loads the tile at the stream position into buffer `buf` and advances the position.
+  // Where the K/V rows of the current (batch, head) lie, set per segment: per KV segment the
+  // pointers to its first rows, the row strides in bytes (below 2^24) and its number of keys.
+  const T* kv_k1;
+  const T* kv_v1;
+  const T* kv_k2;
+  const T* kv_v2;
+  unsigned kss1, vss1, kss2, vss2;
+  int keys1, keys2;
+  // Loads KV tile t of the current (batch, head) into buffer `buf`.
   auto issue_tile = [&](int t, int buf) {
     if ((kWaves == LW || wave < LW) && ld_on) {
-      const int last = (ld_left < kKeysPerTile ? ld_left : kKeysPerTile) - 1;
+      const bool second = t >= nt1;
+      const unsigned row0 = (unsigned)(second ? t - nt1 : t) * kKeysPerTile;   // first key of the tile within its segment
+      const unsigned kss = second ? kss2 : kss1, vss = second ? vss2 : vss1;
+      const T* kp = (const T*)((const unsigned char*)(second ? kv_k2 : kv_k1) + (uint64_t)row0 * kss);
+      const T* vp = (const T*)((const unsigned char*)(second ? kv_v2 : kv_v1) + (uint64_t)row0 * vss);
+      const int left = (second ? keys2 : keys1) - (int)row0;
+      const int last = (left < kKeysPerTile ? left : kKeysPerTile) - 1;
       const unsigned bo = buf * G::BUF_BYTES;
 #pragma unroll
       for (int i = 0; i < PAIRS; i++) {
         int r = ld_row0 + LW * i;
         r = r < last ? r : last;  // rows past the end of the segment re-read its last row
-        load_lds_16(ld_kp, __umul24((unsigned)r, ld_kss) + ld_colb, ld_kdst + bo + i * LW * G::K_PITCH);
-        load_lds_16(ld_vp, __umul24((unsigned)r, ld_vss) + ld_colb, ld_vdst + bo + i * LW * G::V_PITCH);
+        load_lds_16(kp, __umul24((unsigned)r, kss) + ld_colb, ld_kdst + bo + i * LW * G::K_PITCH);
+        load_lds_16(vp, __umul24((unsigned)r, vss) + ld_colb, ld_vdst + bo + i * LW * G::V_PITCH);
       }
-    }
-    if (t + 1 == nt1) {
-      seek_tile(t + 1);
-    } else {
-      ld_kp += ld_kstep; ld_vp += ld_vstep; ld_left -= kKeysPerTile;
     }
   };
 
   // ---- LDS read addresses: one per-lane base each for K and V, the rest are immediates ------
   // K fragment (A operand of S^T) for key block kb, step ks: row 32kb + l32, bytes 32ks + 16hh.
   //   row -> piece (row % NG), slot (row / NG)
-  const int kbase_off = (l32 % G::NG) * G::K_PITCH + (l32 / G::NG) * G::ROW_BYTES + hh * 16;
+  unsigned kbase_off = lds_base + (l32 % G::NG) * G::K_PITCH + (l32 / G::NG) * G::ROW_BYTES + hh * 16;
+  asm volatile("" : "+v"(kbase_off));  // one register, not its summands, lives through the loop
   constexpr int K_KB_STEP = (32 / G::NG) * G::ROW_BYTES;  // +32 rows = +32/NG slots
   // V^T fragment (A operand of O^T) for d block db, key step j (16 keys), half rd (keys +0 / +8):
   // as a SOURCE lane of the transposed read, lane (group g = lane/16, s = lane%16) supplies the
   // 8 bytes at key row 16j + 8rd + 4hh + s/4, elements d = 32db + 16(g%2) + 4(s%4) .. +3; the
   // read returns to lane (g, i) the four keys of that row group at d = 32db + 16(g%2) + i.
   const int vsrc_row = 4 * hh + ((lane & 15) >> 2);  // row within the 16-key step, rd = 0
-  const int vbase_off = (vsrc_row % G::NG) * G::V_PITCH + (vsrc_row / G::NG) * G::ROW_BYTES +
-                        (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  unsigned vbase_off = lds_base + G::K_BYTES + (vsrc_row % G::NG) * G::V_PITCH + (vsrc_row / G::NG) * G::ROW_BYTES +
+                       (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  asm volatile("" : "+v"(vbase_off));
   // +8 rows (rd) and +16 rows (j): both keep row % NG pattern simple because NG is 8 or 16.
   constexpr int V_RD_STEP = (G::NG == 16) ? 8 * G::V_PITCH : G::ROW_BYTES;  // NG=8: +8 rows = +1 slot
   constexpr int V_J_STEP = (16 / G::NG) * G::ROW_BYTES;
 
-  // ---- online softmax state: one query per lane (both halves of the wavefront agree) ------
-  const float c = p.scale * kLog2e;  // logits are kept in log2 units
-  float m_used = -INFINITY;          // running (lazily updated) row maximum of the raw dot products
-  float l_part = 0.f;                // this lane's share of the running row sum
-  f32x16 oacc[DBLOCKS];
-#pragma unroll
-  for (int db = 0; db < DBLOCKS; db++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+  const float c = pp->scale * kLog2e;  // logits are kept in log2 units
 
-  if (PAD) {  // zero the columns that no load writes (all of both buffers: simplest)
+  if (PAD) {  // zero the columns that no load writes (all of both buffers: simplest); once per workgroup
     typedef __attribute__((ext_vector_type(4))) int i32x4;
     const i32x4 zero = {0, 0, 0, 0};
-    for (int i = tid * 16; i < 2 * G::BUF_BYTES; i += 64 * kWaves * 16) *(XDIT_LDS i32x4*)((XDIT_LDS unsigned char*)smem + i) = zero;
+    for (int i = (wave * 64 + lane) * 16; i < 2 * G::BUF_BYTES; i += 64 * kWaves * 16) *(XDIT_LDS i32x4*)((XDIT_LDS unsigned char*)smem + i) = zero;
     __syncthreads();
   }
-  seek_tile(it0);
-  issue_tile(it0, 0);
-  // Make the compiler account for the Q fragment loads here, before the loop: the tile loads
-  // above are invisible to its outstanding-load bookkeeping, so any wait it placed for a Q
-  // fragment inside the loop would also wait for the prefetch of the next tile.
-#pragma unroll
-  for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+v"(qf[ks]));
 
-  for (int t = it0; t < it1; t++) {
-    const int buf = (t - it0) & 1;
-    // Tile t has landed (this thread's loads) and, after the barrier, everyone's; the barrier
-    // also means every wavefront is done reading the other buffer, which tile t+1 now overwrites.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (t + 1 < it1) issue_tile(t + 1, buf ^ 1);
-
-    const XDIT_LDS unsigned char* ktile =
-        (const XDIT_LDS unsigned char*)(smem + buf * G::BUF_BYTES) + kbase_off;
-    const XDIT_LDS unsigned char* vtile =
-        (const XDIT_LDS unsigned char*)(smem + buf * G::BUF_BYTES + G::K_BYTES) + vbase_off;
-
-    // ---- S^T = K Q^T : 2 blocks of 32 keys x 32 queries ---------------------------------
-    f32x16 sacc[2];
-    {
-      constexpr int PD = kPrefetch;   // K fragment reads in flight
-      constexpr int NR = 2 * KSTEPS;  // reads (= MFMAs) of this product
-      const unsigned kaddr = (unsigned)(uintptr_t)ktile;
-      vec8 kf[NR];
-      static_for<PD>([&](auto I) {
-        constexpr int i = I;
-        lds_read_b128<(i / KSTEPS) * K_KB_STEP + (i % KSTEPS) * 32>(kf[i], kaddr);
-      });
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
-      static_for<NR>([&](auto I) {
-        constexpr int i = I;
-        constexpr int younger = (i + PD <= NR ? PD : NR - i) - 1;
-        lds_wait<younger>(kf[i]);
-        sacc[i / KSTEPS] = Mfma16<T>::mma(kf[i], qf[i % KSTEPS], sacc[i / KSTEPS]);
-        if constexpr (i + PD < NR) {
-          constexpr int n = i + PD;
-          lds_read_b128<(n / KSTEPS) * K_KB_STEP + (n % KSTEPS) * 32>(kf[n], kaddr);
-        }
-      });
-    }
-    // ---- mask keys past the end of the segment (only its last tile can be partial) -------
-    const int valid = (t < nt1) ? p.Sk - t * kKeysPerTile : p.Sk2 - (t - nt1) * kKeysPerTile;
-    if (valid < kKeysPerTile) {
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          int key = 32 * kb + 8 * (i >> 2) + 4 * hh + (i & 3);
-          if (key >= valid) sacc[kb][i] = -INFINITY;
-        }
-    }
-
-    // ---- online softmax ---------------------------------------------------------------
-    float mx = sacc[0][0];
-#pragma unroll
-    for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[0][i]);
-#pragma unroll
-    for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[1][i]);
-    mx = max_halves(mx);
-    const float m_new = fmaxf(m_used, mx);
-    const bool grow = (m_new - m_used) * c > kLazyRescaleLog2;  // true on the first tile (-inf)
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-      const float alpha = fast_exp2((m_used - m_new) * c);  // 0 on the first tile
-      m_used = m_new;
-      l_part *= alpha;
-#pragma unroll
-      for (int db = 0; db < DBLOCKS; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-    }
-    const float mc = m_used * c;
-    vec8 pf[4];  // P^T as B operands: pf[j] = keys 16j..16j+15 of this tile (permuted inside)
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-      for (int i = 0; i < 16; i += 2) {
-        float p0 = fast_exp2(__builtin_fmaf(sacc[kb][i], c, -mc));
-        float p1 = fast_exp2(__builtin_fmaf(sacc[kb][i + 1], c, -mc));
-        l_part += p0 + p1;
-        f32x2 pp = {p0, p1};
-        vec2 pk = __builtin_convertvector(pp, vec2);
-        const int j = 2 * kb + (i >> 3);
-        pf[j][(i & 7)] = pk[0];
-        pf[j][(i & 7) + 1] = pk[1];
-      }
-    }
-
-    // ---- O^T += V^T P^T ------------------------------------------------------------------
-    {
-      constexpr int PD = kPrefetch;  // MFMAs whose two V^T reads are in flight
-      constexpr int NM = 4 * DBLOCKS;
-      typedef __attribute__((ext_vector_type(8))) short s16x8;
-      const unsigned vaddr = (unsigned)(uintptr_t)vtile;
-      s16x4 v0[NM], v1[NM];
-      static_for<PD>([&](auto I) {
-        constexpr int i = I;
-        constexpr int off = (i / DBLOCKS) * V_J_STEP + (i % DBLOCKS) * 64;
-        lds_read_tr16_b64<off>(v0[i], vaddr);
-        lds_read_tr16_b64<off + V_RD_STEP>(v1[i], vaddr);
-      });
-      static_for<NM>([&](auto I) {
-        constexpr int i = I;
-        constexpr int younger = 2 * ((i + PD <= NM ? PD : NM - i) - 1);
-        lds_wait2<younger>(v0[i], v1[i]);
-        s16x8 vv = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3, 4, 5, 6, 7);
-        oacc[i % DBLOCKS] = Mfma16<T>::mma(__builtin_bit_cast(vec8, vv), pf[i / DBLOCKS], oacc[i % DBLOCKS]);
-        if constexpr (i + PD < NM) {
-          constexpr int n = i + PD;
-          constexpr int off = (n / DBLOCKS) * V_J_STEP + (n % DBLOCKS) * 64;
-          lds_read_tr16_b64<off>(v0[n], vaddr);
-          lds_read_tr16_b64<off + V_RD_STEP>(v1[n], vaddr);
-        }
-      });
-    }
-  }
-
-  // ---- epilogue -----------------------------------------------------------------------------
-  const float l_tot = sum_halves(l_part);
-  const float inv = 1.0f / l_tot;
-  const float lse = (m_used * c + fast_log2(l_tot)) * kLn2;
-  if constexpr (!FUSED) {
-    // The normalised rows go out through LDS, 64 columns at a time: lane (query, half) writes
-    // its 4-element pieces into a [32 rows][64 columns] block private to the wavefront, which is
-    // read back with 8 lanes per row, so that every global store covers whole 128-byte lines of
-    // 8 rows (stored straight from the accumulator layout, a store touches 32 rows 16 bytes at
-    // a time and the epilogue is bound by the number of memory requests).
-    typedef __attribute__((ext_vector_type(4))) T vec4;
-    __syncthreads();  // every wavefront is done with the fragments of the last tile
-    XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + wave * kStageBytes;
-    const int row0 = qt * kRowsPerBlock + wave * kRowsPerWave;   // first query row of this wavefront
-    T* obase;
-    int64_t ostride;
-    int rows_live = kRowsPerWave;
-    if (part_out != nullptr) {
-      obase = part_out + (int64_t)(wave * kRowsPerWave) * D;
-      ostride = D;
+  // ---- per segment: coordinates, Q fragments (B operand of S^T, lane = (query l32, contraction
+  // half hh)) and the first K/V tile; issued here for the first segment and, for every later
+  // one, ahead of the epilogue of its predecessor -------------------------------------------
+  int b, h, qt;
+  vec8 qf[KSTEPS];
+  auto open_segment = [&](const Segment& sg) {
+    const int lane = lane_now(), l32 = lane & 31, hh = lane >> 5;
+    const int nq_tiles = pp->nq_tiles, H = pp->H;
+    const int bh = sg.tile / nq_tiles;
+    qt = sg.tile - bh * nq_tiles;
+    b = bh / H;
+    h = bh - b * H;
+    kv_k1 = (const T*)pp->k + b * pp->ks_b + h * pp->ks_h;
+    kv_v1 = (const T*)pp->v + b * pp->vs_b + h * pp->vs_h;
+    kss1 = (unsigned)pp->ks_s * 2; vss1 = (unsigned)pp->vs_s * 2;
+    keys1 = pp->Sk; keys2 = pp->Sk2;
+    if (keys2 > 0) {
+      kv_k2 = (const T*)pp->k2 + b * pp->k2s_b + h * pp->k2s_h;
+      kv_v2 = (const T*)pp->v2 + b * pp->v2s_b + h * pp->v2s_h;
+      kss2 = (unsigned)pp->k2s_s * 2; vss2 = (unsigned)pp->v2s_s * 2;
     } else {
-      obase = (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)row0 * p.os_s;
-      ostride = p.os_s;
-      rows_live = p.Sq - row0;  // may be <= 0 or above 32
+      kv_k2 = kv_k1; kv_v2 = kv_v1; kss2 = kss1; vss2 = vss1;
     }
-    const int cols_live = part_out != nullptr ? 32 * DBLOCKS : (PAD ? dact : D);
-    const int rd_row = lane >> 3;          // + 8r
-    const int rd_col = (lane & 7) * 8;     // element column within the 64-column pass
+    const int Sq = pp->Sq;
+    const int qrow = qt * kRowsPerBlock + wave * kRowsPerWave + l32;
+    const int qrow_c = qrow < Sq ? qrow : Sq - 1;
+    const T* qptr = (const T*)pp->q + b * pp->qs_b + h * pp->qs_h + (int64_t)qrow_c * pp->qs_s + hh * 8;
 #pragma unroll
-    for (int half = 0; half < (DBLOCKS + 1) / 2; half++) {
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      if (!PAD || ks * 16 + hh * 8 < dact) {
+        qf[ks] = *(const vec8*)(qptr + ks * 16);
+      } else {
 #pragma unroll
-      for (int dbl = 0; dbl < 2; dbl++) {
-        const int db = 2 * half + dbl;
-        if (db < DBLOCKS) {
+        for (int e = 0; e < 8; e++) qf[ks][e] = (T)0.f;
+      }
+    }
+    issue_tile(sg.it0, 0);
+  };
+  XDIT_TRACE_POINT(seg.slot >= 0, 0);
+  open_segment(seg);
+
+  for (;;) {  // segments of this workgroup
+    // Coordinates of the segment being computed (open_segment of the next one overwrites them).
+    const int cb = b, ch = h, cqt = qt;
+    T* part_out = nullptr;
+    float* part_lse = nullptr;
+    if (seg.slot >= 0) {
+      part_out = (T*)pp->ws_out + seg.slot * kRowsPerBlock * D;
+      part_lse = pp->ws_lse + seg.slot * kRowsPerBlock;
+    }
+    // Streamed sharing: stream position i holds KV tile it0 + i while i < n_own; later positions
+    // are drawn from the tile's counter, two positions ahead of their use.
+    const int n_own = seg.it1 - seg.it0;
+    const bool streamed = seg.dyn >= 0;
+    const int pool_len = nt - seg.pool0;
+    unsigned* const draw_counter = streamed ? pp->split_counter + seg.dyn : nullptr;
+    bool pool_open = streamed;  // thread 0: no ticket has come back past the end of the pool yet
+    const int keys_1 = keys1, keys_2 = keys2;
+
+    // ---- online softmax state: one query per lane (both halves of the wavefront agree) ------
+    float m_used = -INFINITY;          // running (lazily updated) row maximum of the raw dot products
+    float l_part = 0.f;                // this lane's share of the running row sum
+    f32x16 oacc[DBLOCKS];
 #pragma unroll
-          for (int a = 0; a < 4; a++) {
-            // registers 4a..4a+3 are d = 32db + 8a + 4hh + 0..3 of this lane's query
-            f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
-                       oacc[db][4 * a + 3] * inv};
-            *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+    for (int db = 0; db < DBLOCKS; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+
+    // Make the compiler account for the Q fragment loads here, before the loop: the tile loads
+    // are invisible to its outstanding-load bookkeeping, so any wait it placed for a Q fragment
+    // inside the loop would also wait for the prefetch of the next tile.
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+v"(qf[ks]));
+
+    int t = seg.it0;
+    for (int i = 0;; i++) {
+      const int buf = i & 1;
+      // Tile t has landed (this thread's loads) and, after the barrier, everyone's; the barrier
+      // also means every wavefront is done reading the other buffer, which the next tile now
+      // overwrites.  A ticket drawn during the previous iteration has come back as well: thread
+      // 0 posts the KV tile it stands for (position i + 1) before the barrier.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (i == 0) { XDIT_TRACE_POINT(seg.slot >= 0, 1); }
+      int t_next;
+      if (i + 1 < n_own) t_next = t + 1;
+      else if (streamed) t_next = __builtin_amdgcn_readfirstlane(drawn[(i + 1) & 1]);  // posted during the previous iteration
+      else t_next = -1;
+      if (t_next >= 0) issue_tile(t_next, buf ^ 1);
+      // Streamed sharing: thread 0 draws the ticket of position i + 2 now and posts the KV tile
+      // it stands for at the end of this iteration, when the ticket has long come back.
+      const bool drawing = streamed && i + 2 >= n_own && t_next >= 0;
+      unsigned draw = 0xffffffffu;
+      if (drawing && wave == 0 && pool_open && lane_now() == 0) draw = draw_ticket(draw_counter);
+
+      const unsigned kaddr = kbase_off + buf * G::BUF_BYTES;
+      const unsigned vaddr = vbase_off + buf * G::BUF_BYTES;
+
+      // ---- S^T = K Q^T : 2 blocks of 32 keys x 32 queries ---------------------------------
+      f32x16 sacc[2];
+      {
+        constexpr int PD = kPrefetch;   // K fragment reads in flight
+        constexpr int NR = 2 * KSTEPS;  // reads (= MFMAs) of this product
+        vec8 kf[NR];
+        static_for<PD>([&](auto I) {
+          constexpr int i_ = I;
+          lds_read_b128<(i_ / KSTEPS) * K_KB_STEP + (i_ % KSTEPS) * 32>(kf[i_], kaddr);
+        });
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+          for (int e = 0; e < 16; e++) sacc[kb][e] = 0.f;
+        static_for<NR>([&](auto I) {
+          constexpr int i_ = I;
+          constexpr int younger = (i_ + PD <= NR ? PD : NR - i_) - 1;
+          lds_wait<younger>(kf[i_]);
+          sacc[i_ / KSTEPS] = Mfma16<T>::mma(kf[i_], qf[i_ % KSTEPS], sacc[i_ / KSTEPS]);
+          if constexpr (i_ + PD < NR) {
+            constexpr int n = i_ + PD;
+            lds_read_b128<(n / KSTEPS) * K_KB_STEP + (n % KSTEPS) * 32>(kf[n], kaddr);
           }
+        });
+      }
+      // ---- mask keys past the end of the segment (only its last tile can be partial) -------
+      const int valid = (t < nt1) ? keys_1 - t * kKeysPerTile : keys_2 - (t - nt1) * kKeysPerTile;
+      if (valid < kKeysPerTile) {
+        const int hh = lane_now() >> 5;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            int key = 32 * kb + 8 * (e >> 2) + 4 * hh + (e & 3);
+            if (key >= valid) sacc[kb][e] = -INFINITY;
+          }
+      }
+
+      // ---- online softmax ---------------------------------------------------------------
+      float mx = sacc[0][0];
+#pragma unroll
+      for (int e = 1; e < 16; e++) mx = fmaxf(mx, sacc[0][e]);
+#pragma unroll
+      for (int e = 0; e < 16; e++) mx = fmaxf(mx, sacc[1][e]);
+      mx = max_halves(mx);
+      const float m_new = fmaxf(m_used, mx);
+      const bool grow = (m_new - m_used) * c > kLazyRescaleLog2;  // true on the first tile (-inf)
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        const float alpha = fast_exp2((m_used - m_new) * c);  // 0 on the first tile
+        m_used = m_new;
+        l_part *= alpha;
+#pragma unroll
+        for (int db = 0; db < DBLOCKS; db++)
+#pragma unroll
+          for (int e = 0; e < 16; e++) oacc[db][e] *= alpha;
+      }
+      const float mc = m_used * c;
+      vec8 pf[4];  // P^T as B operands: pf[j] = keys 16j..16j+15 of this tile (permuted inside)
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) {
+          float p0 = fast_exp2(__builtin_fmaf(sacc[kb][e], c, -mc));
+          float p1 = fast_exp2(__builtin_fmaf(sacc[kb][e + 1], c, -mc));
+          l_part += p0 + p1;
+          f32x2 pp = {p0, p1};
+          vec2 pk = __builtin_convertvector(pp, vec2);
+          const int j = 2 * kb + (e >> 3);
+          pf[j][(e & 7)] = pk[0];
+          pf[j][(e & 7) + 1] = pk[1];
         }
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int row = rd_row + 8 * r;
-        const int col = 64 * half + rd_col;
-        const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
-        if (row < rows_live && col < cols_live) *(vec8*)(obase + row * ostride + col) = x;
+
+      // ---- O^T += V^T P^T ------------------------------------------------------------------
+      {
+        constexpr int PD = kPrefetch;  // MFMAs whose two V^T reads are in flight
+        constexpr int NM = 4 * DBLOCKS;
+        typedef __attribute__((ext_vector_type(8))) short s16x8;
+        s16x4 v0[NM], v1[NM];
+        static_for<PD>([&](auto I) {
+          constexpr int i_ = I;
+          constexpr int off = (i_ / DBLOCKS) * V_J_STEP + (i_ % DBLOCKS) * 64;
+          lds_read_tr16_b64<off>(v0[i_], vaddr);
+          lds_read_tr16_b64<off + V_RD_STEP>(v1[i_], vaddr);
+        });
+        static_for<NM>([&](auto I) {
+          constexpr int i_ = I;
+          constexpr int younger = 2 * ((i_ + PD <= NM ? PD : NM - i_) - 1);
+          lds_wait2<younger>(v0[i_], v1[i_]);
+          s16x8 vv = __builtin_shufflevector(v0[i_], v1[i_], 0, 1, 2, 3, 4, 5, 6, 7);
+          oacc[i_ % DBLOCKS] = Mfma16<T>::mma(__builtin_bit_cast(vec8, vv), pf[i_ / DBLOCKS], oacc[i_ % DBLOCKS]);
+          if constexpr (i_ + PD < NM) {
+            constexpr int n = i_ + PD;
+            constexpr int off = (n / DBLOCKS) * V_J_STEP + (n % DBLOCKS) * 64;
+            lds_read_tr16_b64<off>(v0[n], vaddr);
+            lds_read_tr16_b64<off + V_RD_STEP>(v1[n], vaddr);
+          }
+        });
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+      if (drawing && wave == 0 && lane_now() == 0) {
+        const bool in_pool = draw < (unsigned)pool_len;
+        drawn[i & 1] = in_pool ? seg.pool0 + (int)draw : -1;   // position i + 2
+        pool_open = in_pool;
+      }
+      if (t_next < 0) break;
+      t = t_next;
     }
-    if (hh == 0 && qrow < p.Sq) {
-      if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
-      else if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = lse;
+    XDIT_TRACE_POINT(seg.slot >= 0, 2);
+    asm volatile("" : "+s"(pp));  // from here on the kernel arguments are read afresh
+
+    // ---- what comes next for this workgroup --------------------------------------------------
+    Segment next_seg;
+    bool more;
+    {
+      const WalkGeom g = walk_geom(pp);
+      unsigned* const range_counter = pp->split_counter;
+      if (walk.wants_claim(range_counter != nullptr && g.split_dyn == 0)) {
+        __syncthreads();  // everyone has read the ticket of the previous claim
+        if (wave == 0 && lane_now() == 0) ticket = atomicAdd(range_counter, 1u);
+        __syncthreads();
+        walk.claimed(g, (unsigned)__builtin_amdgcn_readfirstlane((int)ticket));
+      }
+      more = walk.next(g, nt, next_seg);
     }
-  } else {
-    // Ring step: fold this block into the fp32 accumulator (the arithmetic of the merge kernel
-    // on the block rounded to T, so the result equals forward + merge bit for bit).  The block
-    // goes through the same LDS transpose as above, so that the accumulator is read and written
-    // in whole rows; the weight of each row's fold travels with it.
-    typedef __attribute__((ext_vector_type(4))) T vec4;
-    __syncthreads();  // every wavefront is done with the fragments of the last tile
-    XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + wave * kStageBytes;
-    XDIT_LDS float* wrow = (XDIT_LDS float*)(stage + kRowsPerWave * kStagePitch);
-    const int row0 = qt * kRowsPerBlock + wave * kRowsPerWave;
-    const bool first = p.acc_first != 0;
-    float* alp = p.acc_lse + b * p.al_b + h * p.al_h + (int64_t)qrow * p.al_s;
-    float w = 0.f, new_lse = lse;
-    if (!first && qrow < p.Sq) {
-      const float la = *alp;
-      w = sigmoid(lse - la);
-      new_lse = la - log_sigmoid(la - lse);
+    __syncthreads();  // every wavefront is done with the K/V fragments of the last tile
+    if (more) {
+      XDIT_TRACE_POINT(next_seg.slot >= 0, 0);
+      open_segment(next_seg);  // Q fragments and first K/V tile (buffer 0) of the next segment
     }
-    if (hh == 0) wrow[l32] = w;
-    float* abase = p.acc_out + b * p.ao_b + h * p.ao_h + (int64_t)row0 * p.ao_s;
-    T* obase = p.out != nullptr ? (T*)p.out + b * p.os_b + h * p.os_h + (int64_t)row0 * p.os_s : nullptr;
-    const int rows_live = p.Sq - row0;
-    const int cols_live = PAD ? dact : D;
-    const int rd_row = lane >> 3;
-    const int rd_col = (lane & 7) * 8;
+
+    // ---- epilogue -----------------------------------------------------------------------------
+    const int lane = lane_now(), l32 = lane & 31, hh = lane >> 5;
+    const int cqrow = cqt * kRowsPerBlock + wave * kRowsPerWave + l32;
+    const float l_tot = sum_halves(l_part);
+    const float inv = 1.0f / l_tot;
+    const float lse = (m_used * c + fast_log2(l_tot)) * kLn2;
+    XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + G::BUF_BYTES + wave * kStageBytes;
+    const int row0 = cqt * kRowsPerBlock + wave * kRowsPerWave;   // first query row of this wavefront
+    if constexpr (!FUSED) {
+      // The normalised rows go out through LDS, 64 columns at a time: lane (query, half) writes
+      // its 4-element pieces into a [32 rows][64 columns] block private to the wavefront, which is
+      // read back with 8 lanes per row, so that every global store covers whole 128-byte lines of
+      // 8 rows (stored straight from the accumulator layout, a store touches 32 rows 16 bytes at
+      // a time and the epilogue is bound by the number of memory requests).
+      typedef __attribute__((ext_vector_type(4))) T vec4;
+      T* obase;
+      int64_t ostride;
+      int rows_live = kRowsPerWave;
+      if (part_out != nullptr) {
+        obase = part_out + (int64_t)(wave * kRowsPerWave) * D;
+        ostride = D;
+      } else {
+        obase = (T*)pp->out + cb * pp->os_b + ch * pp->os_h + (int64_t)row0 * pp->os_s;
+        ostride = pp->os_s;
+        rows_live = pp->Sq - row0;  // may be <= 0 or above 32
+      }
+      const int cols_live = part_out != nullptr ? 32 * DBLOCKS : (PAD ? dact : D);
+      const int rd_row = lane >> 3;          // + 8r
+      const int rd_col = (lane & 7) * 8;     // element column within the 64-column pass
 #pragma unroll
-    for (int half = 0; half < (DBLOCKS + 1) / 2; half++) {
+      for (int half = 0; half < (DBLOCKS + 1) / 2; half++) {
 #pragma unroll
-      for (int dbl = 0; dbl < 2; dbl++) {
-        const int db = 2 * half + dbl;
-        if (db < DBLOCKS) {
+        for (int dbl = 0; dbl < 2; dbl++) {
+          const int db = 2 * half + dbl;
+          if (db < DBLOCKS) {
 #pragma unroll
-          for (int a = 0; a < 4; a++) {
-            f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
-                       oacc[db][4 * a + 3] * inv};
-            *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+            for (int a = 0; a < 4; a++) {
+              // registers 4a..4a+3 are d = 32db + 8a + 4hh + 0..3 of this lane's query
+              f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                         oacc[db][4 * a + 3] * inv};
+              *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+            }
           }
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int row = rd_row + 8 * r;
+          const int col = 64 * half + rd_col;
+          const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
+          // streaming stores: the rows are not read again by this kernel, and lines that leave the
+          // cache as they are written are not left for the write-back at the kernel's end
+          if (row < rows_live && col < cols_live) __builtin_nontemporal_store(x, (vec8*)(obase + row * ostride + col));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+      if (hh == 0 && cqrow < pp->Sq) {
+        if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
+        else if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = lse;
+      }
+    } else {
+      // Ring step: fold this block into the fp32 accumulator (the arithmetic of the merge kernel
+      // on the block rounded to T, so the result equals forward + merge bit for bit).  The block
+      // goes through the same LDS transpose as above, so that the accumulator is read and written
+      // in whole rows; the weight of each row's fold travels with it.
+      typedef __attribute__((ext_vector_type(4))) T vec4;
+      XDIT_LDS float* wrow = (XDIT_LDS float*)(stage + kRowsPerWave * kStagePitch);
+      const bool first = pp->acc_first != 0;
+      float* alp = pp->acc_lse + cb * pp->al_b + ch * pp->al_h + (int64_t)cqrow * pp->al_s;
+      float w = 0.f, new_lse = lse;
+      if (!first && cqrow < pp->Sq) {
+        const float la = *alp;
+        w = sigmoid(lse - la);
+        new_lse = la - log_sigmoid(la - lse);
+      }
+      if (hh == 0) wrow[l32] = w;
+      float* abase = pp->acc_out + cb * pp->ao_b + ch * pp->ao_h + (int64_t)row0 * pp->ao_s;
+      T* obase = pp->out != nullptr ? (T*)pp->out + cb * pp->os_b + ch * pp->os_h + (int64_t)row0 * pp->os_s : nullptr;
+      const int rows_live = pp->Sq - row0;
+      const int cols_live = PAD ? dact : D;
+      const int rd_row = lane >> 3;
+      const int rd_col = (lane & 7) * 8;
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int row = rd_row + 8 * r;
-        const int col = 64 * half + rd_col;
-        const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
-        const float wr = wrow[row];
-        if (row < rows_live && col < cols_live) {
-          float* aptr = abase + row * p.ao_s + col;
-          f32x4 m0, m1;
+      for (int half = 0; half < (DBLOCKS + 1) / 2; half++) {
 #pragma unroll
-          for (int e = 0; e < 4; e++) { m0[e] = (float)x[e]; m1[e] = (float)x[4 + e]; }
-          if (!first) {
-            const f32x4 a0 = *(const f32x4*)aptr, a1 = *(const f32x4*)(aptr + 4);
+        for (int dbl = 0; dbl < 2; dbl++) {
+          const int db = 2 * half + dbl;
+          if (db < DBLOCKS) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) { m0[e] = fold_value(a0[e], m0[e], wr); m1[e] = fold_value(a1[e], m1[e], wr); }
-          }
-          if (p.acc_store) { *(f32x4*)aptr = m0; *(f32x4*)(aptr + 4) = m1; }
-          if (obase != nullptr) {
-            vec8 y;
-#pragma unroll
-            for (int e = 0; e < 4; e++) { y[e] = (T)m0[e]; y[4 + e] = (T)m1[e]; }
-            *(vec8*)(obase + row * p.os_s + col) = y;
+            for (int a = 0; a < 4; a++) {
+              f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                         oacc[db][4 * a + 3] * inv};
+              *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+            }
           }
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int row = rd_row + 8 * r;
+          const int col = 64 * half + rd_col;
+          const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
+          const float wr = wrow[row];
+          if (row < rows_live && col < cols_live) {
+            float* aptr = abase + row * pp->ao_s + col;
+            f32x4 m0, m1;
+#pragma unroll
+            for (int e = 0; e < 4; e++) { m0[e] = (float)x[e]; m1[e] = (float)x[4 + e]; }
+            if (!first) {
+              const f32x4 a0 = *(const f32x4*)aptr, a1 = *(const f32x4*)(aptr + 4);
+#pragma unroll
+              for (int e = 0; e < 4; e++) { m0[e] = fold_value(a0[e], m0[e], wr); m1[e] = fold_value(a1[e], m1[e], wr); }
+            }
+            if (pp->acc_store) { *(f32x4*)aptr = m0; *(f32x4*)(aptr + 4) = m1; }
+            if (obase != nullptr) {
+              vec8 y;
+#pragma unroll
+              for (int e = 0; e < 4; e++) { y[e] = (T)m0[e]; y[4 + e] = (T)m1[e]; }
+              *(vec8*)(obase + row * pp->os_s + col) = y;
+            }
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+      if (hh == 0 && cqrow < pp->Sq) {
+        *alp = new_lse;
+        if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = new_lse;
+      }
     }
-    if (hh == 0 && qrow < p.Sq) {
-      *alp = new_lse;
-      if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = new_lse;
+    XDIT_TRACE_POINT(seg.slot >= 0, 3);
+    if (!more) break;
+    if (PAD) {  // the staging blocks lay over the second K/V buffer: clear it again (the barrier of the first iteration orders this)
+      typedef __attribute__((ext_vector_type(4))) int i32x4;
+      const i32x4 zero = {0, 0, 0, 0};
+      for (int i = (wave * 64 + lane) * 16; i < G::BUF_BYTES; i += 64 * kWaves * 16) *(XDIT_LDS i32x4*)((XDIT_LDS unsigned char*)smem + G::BUF_BYTES + i) = zero;
     }
+    seg = next_seg;
   }
 }
 
 template <typename T, int D, int DC, int NW, bool PAD, bool FUSED>
 __global__ __launch_bounds__(64 * NW, NW == 12 ? 3 : 2) void attn_fwd_16_kernel(const AttnParams p) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // 2 x [K tile | V tile]
-  run_workgroup<T, kRowsPerWave * NW, D>(p, [&](int tile, int it0, int it1, T* part_out, float* part_lse) {
-    attn_segment<T, D, DC, NW, PAD, FUSED>(p, smem, tile, it0, it1, part_out, part_lse);
-  });
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // [K tile | V tile] [K tile | V tile, or output staging]
+  attn_workgroup<T, D, DC, NW, PAD, FUSED>(smem);
 }
 
 // Workgroups of NW wavefronts resident at once: LDS and registers allow two 4-wavefront
@@ -462,7 +591,7 @@ static int resident_workgroups(int NW, int planned_cus) { return resident_cus(pl
 template <typename T, int D, int DC, int NW, bool PAD, bool FUSED>
 static hipError_t launch_kernel(const AttnParams& q, hipStream_t stream) {
   static std::atomic<bool> lds_ready[kMaxDevices];
-  constexpr int lds = 2 * TileGeom<D>::BUF_BYTES > NW * kStageBytesPerWave ? 2 * TileGeom<D>::BUF_BYTES : NW * kStageBytesPerWave;
+  constexpr int lds = lds_bytes_16<D, NW>();
   const int slot = current_device_slot();
   if (!lds_ready[slot].load(std::memory_order_relaxed)) {  // > 64 KiB of dynamic LDS must be enabled once per kernel and device
     hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_16_kernel<T, D, DC, NW, PAD, FUSED>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -481,9 +610,9 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
   // the ring step folds in the epilogue of whole query tiles: no shared last round
-  bind_workspace(q, p, FUSED ? 0 : plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, kClaimsPerWorkgroup), rows, D, 2);
+  bind_workspace(q, p, FUSED ? 0 : plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, kClaimsPerWorkgroup, true), rows, D, 2);
   if constexpr (!FUSED) {
-    if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
+    launch_counter_reset(q, stream);
   }
   if (q.d_actual == D) q.d_actual = 0;
   // computed head_dims built for tensors smaller than D: 80, 96, 112 (and 128) of 128; 32 (and 64) of 64
@@ -503,7 +632,7 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
     if (q.split_units) {
       const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
       const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
-      hipLaunchKernelGGL((attn_combine_kernel<T, D>), cgrid, dim3(256), 0, stream, q, rows, nt);
+      hipLaunchKernelGGL((attn_combine_kernel<T, D>), cgrid, dim3(256), 0, stream, q, rows, nt, split_counters(q));
     }
   }
   return hipGetLastError();

@@ -329,13 +329,13 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
   bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1), rows, D, 2);
-  if (q.split_counter != nullptr) hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(64), 0, stream, q.split_counter);
+  launch_counter_reset(q, stream);
   dim3 grid(split_grid(q));
   hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW>), grid, dim3(64 * NW), 0, stream, q);
   if (q.split_units) {
     const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
     const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
-    hipLaunchKernelGGL((attn_combine_kernel<TO, D>), cgrid, dim3(256), 0, stream, q, rows, nt);
+    hipLaunchKernelGGL((attn_combine_kernel<TO, D>), cgrid, dim3(256), 0, stream, q, rows, nt, split_counters(q));
   }
   return hipGetLastError();
 }

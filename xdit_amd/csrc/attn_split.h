@@ -41,10 +41,10 @@ __device__ __forceinline__ void run_workgroup(const AttnParams& p, Seg seg) {
   }
 }
 
-// Clears the range counter of a balanced launch (a kernel, not a memset, so that the sequence
-// can be captured into a graph).
-static __global__ void attn_counter_reset_kernel(unsigned* counter) {
-  if (threadIdx.x == 0) *counter = 0u;
+// Clears the counters of a balanced launch (a kernel, not a memset, so that the sequence can be
+// captured into a graph).
+static __global__ void attn_counter_reset_kernel(unsigned* counter, int n) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) counter[i] = 0u;
 }
 
 // Folds the parts of every query tile that was split: out = sum_k exp(lse_k - L) out_k,
@@ -52,10 +52,13 @@ static __global__ void attn_counter_reset_kernel(unsigned* counter) {
 // grid = (ceil(rows_per_block * D/8 / 256), shared query tiles): blockIdx.y is the tile, so the
 // tile's coordinates and part range are wavefront-uniform.
 template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, const int rows_per_block, const int nt) {
+__global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, const int rows_per_block, const int nt, const int counters) {
   constexpr int TPR = D / 8;
   const int r = blockIdx.y;  // which of the shared query tiles
   const int local = blockIdx.x * 256 + threadIdx.x;
+  // the counters the attention kernel used go back to zero, for the next call on this workspace
+  if (blockIdx.x == 0 && blockIdx.y == 0)
+    for (int i = threadIdx.x; i < counters; i += 256) p.ws_counters[i] = 0u;
   const int row = local / TPR;
   const int col = (local - row * TPR) * 8;
   if (row >= rows_per_block) return;
@@ -146,10 +149,29 @@ constexpr int kClaimsPerWorkgroup = 6;
 // the balanced launch needs (0 = plain launch).
 // `rows` query rows per workgroup, `slots` workgroups resident at once, `out_bytes` per output
 // element, `claims` ranges per workgroup to aim at (1: every workgroup gets one range).
-static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int out_bytes, int claims) {
+// A workspace starts with this many bytes of counters (4096 of them), whatever the launch uses of
+// them: partial results never lie there, so counters that one call leaves at zero are still zero
+// for the next call on the same workspace, whatever its shape.
+constexpr size_t kCounterRegionBytes = 16384;
+
+// Iterations a member of a tile's group owns under streamed sharing (the loop needs two to start
+// drawing from the counter without waiting for it).
+constexpr int kStreamedOwn = 2;
+
+// Number of counters a planned launch uses (0: none).
+static inline int split_counters(const AttnParams& q) {
+  if (q.split_dyn) return q.total_tiles - q.split_full;
+  return q.split_units > q.split_claimers ? 1 : 0;
+}
+static inline size_t split_parts_bytes(const AttnParams& q, int rows, int D, int out_bytes) {
+  return (size_t)(q.total_tiles - q.split_full) * q.split_pmax * rows * ((size_t)D * out_bytes + 4);
+}
+
+static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int out_bytes, int claims, bool streamed = false) {
   q.split_units = q.split_full = q.split_len = q.split_pmax = q.split_share = q.split_claimers = 0;
   q.split_fuse0 = 0x7fffffff;
   q.split_counter = nullptr;
+  q.split_dyn = q.split_s0 = 0;
   const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
   const int T = q.total_tiles;
   const int full = (T / slots) * slots;
@@ -162,6 +184,22 @@ static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int o
   // balance only when the saving clearly exceeds the cost of the extra prologues, the partial
   // results and the combine pass (measured: about 10 iterations' worth).
   if (nt - share < 48) return 0;
+  // Few shared tiles with short shares: streamed sharing.  Every resident workgroup joins the
+  // group of one shared tile; unless the caller asks for bit-reproducible results.
+  if (streamed && !q.deterministic && share < 2 * kMinClaimLen && rem * 4 <= slots) {
+    const int pmax = (slots + rem - 1) / rem;
+    if (pmax * kStreamedOwn * 2 <= nt && (size_t)rem * 4 <= kCounterRegionBytes) {
+      q.split_full = full;
+      q.split_units = q.split_claimers = slots;
+      q.split_len = share;
+      q.split_share = share;
+      q.split_pmax = pmax;
+      q.split_fuse0 = full >= slots ? full - slots : 0x7fffffff;
+      q.split_dyn = 1;
+      q.split_s0 = kStreamedOwn;
+      return kCounterRegionBytes + split_parts_bytes(q, rows, D, out_bytes);
+    }
+  }
   // Long shares are cut into several ranges that are claimed one after the other.
   int len = share;
   if (claims > 1 && share >= 2 * kMinClaimLen) {
@@ -177,25 +215,34 @@ static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int o
   q.split_pmax = (nt + len - 1) / len + 1;
   q.split_claimers = claimers;
   q.split_fuse0 = full >= claimers ? full - claimers : 0x7fffffff;
-  const size_t parts = (size_t)rem * q.split_pmax * rows * ((size_t)D * out_bytes + 4);
-  return units > claimers ? ((parts + 255) & ~(size_t)255) + 256 : parts;  // + the range counter
+  return kCounterRegionBytes + split_parts_bytes(q, rows, D, out_bytes);
 }
 
-// Point ws_lse (and the range counter) behind the partial outputs, or fall back to a plain launch
-// when the caller gave no (or too small a) workspace.
+// Lay the workspace out: counters, partial outputs, partial log-sum-exps; or fall back to a plain
+// launch when the caller gave no (or too small a) workspace.
 static inline void bind_workspace(AttnParams& q, const AttnParams& p, size_t need, int rows, int D, int out_bytes) {
   if (need == 0 || p.ws_out == nullptr || p.ws_bytes < need) {
     q.split_units = q.split_full = q.split_len = q.split_pmax = q.split_share = q.split_claimers = 0;
     q.split_fuse0 = 0x7fffffff;
     q.split_counter = nullptr;
+    q.split_dyn = q.split_s0 = 0;
+    q.ws_out = nullptr;
   } else {
     const size_t rem = (size_t)(q.total_tiles - q.split_full);
-    q.ws_lse = (float*)((unsigned char*)p.ws_out + rem * q.split_pmax * rows * D * out_bytes);
-    if (q.split_units > q.split_claimers) {
-      const size_t parts = rem * q.split_pmax * rows * ((size_t)D * out_bytes + 4);
-      q.split_counter = (unsigned*)((unsigned char*)p.ws_out + ((parts + 255) & ~(size_t)255));
-    }
+    q.ws_counters = (unsigned*)p.ws_out;
+    q.ws_out = (unsigned char*)p.ws_out + kCounterRegionBytes;
+    q.ws_lse = (float*)((unsigned char*)q.ws_out + rem * q.split_pmax * rows * D * out_bytes);
+    q.split_counter = split_counters(q) > 0 ? q.ws_counters : nullptr;
   }
+}
+
+// The launches around the attention kernel of a balanced launch.  Counters must be zero when the
+// attention kernel starts: a workspace whose contents the caller vouches for (ws_preserved: left
+// as this library's previous call on it left them) has them at zero already, since the fold
+// kernel clears what its launch used; otherwise a small kernel clears the whole region first.
+static inline void launch_counter_reset(const AttnParams& q, hipStream_t stream) {
+  if (q.split_units != 0 && !q.ws_preserved)
+    hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(256), 0, stream, q.ws_counters, (int)(kCounterRegionBytes / 4));
 }
 
 // Workgroups of a launch planned by plan_split (after bind_workspace).

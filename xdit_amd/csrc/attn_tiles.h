@@ -58,7 +58,7 @@ __device__ __forceinline__ void load_lds_16(const void* base, unsigned off, unsi
       "s_nop 0\n\t"
       "global_load_lds_dwordx4 %1, %2"
       :
-      : "s"(lds), "v"(off), "s"(base)
+      : "s"(__builtin_amdgcn_readfirstlane(lds)), "v"(off), "s"(base)
       : "memory", "m0");
 }
 

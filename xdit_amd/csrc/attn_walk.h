@@ -25,14 +25,19 @@ XDIT_HD int xcd_tile_index(int block, int tiles_per_xcd) {
 // One piece of work of a workgroup: KV iterations [it0, it1) of query tile `tile`.  slot < 0: the
 // workgroup owns the whole tile and writes the final result; otherwise the piece is one part of a
 // query tile whose KV iterations are shared, and its partial result goes to that workspace slot.
+// dyn >= 0: after [it0, it1) the workgroup goes on with KV iterations pool0 + ticket of the same
+// query tile, one at a time, tickets drawn from counter `dyn` of the launch until they run past
+// the tile's last iteration; everything it processes goes into the one partial result of `slot`.
 struct Segment {
   int tile, it0, it1;
   int64_t slot;
+  int dyn, pool0;
 };
 
 // The sequence of segments of workgroup `w`.  P is any struct with the launch-geometry members of
 // AttnParams (total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax,
-// split_fuse0, split_claimers); `nt` is the number of KV iterations of a whole tile.
+// split_fuse0, split_claimers, split_dyn, split_s0); `nt` is the number of KV iterations of a
+// whole tile.
 // Plain launch (split_units == 0): workgroup = one query tile over all KV iterations.  Balanced
 // launch: the first split_full workgroups each take a whole query tile; the KV iterations of the
 // remaining query tiles, laid end to end, are cut into split_units ranges of split_len
@@ -44,6 +49,12 @@ struct Segment {
 // Claimer c starts with range c; when there are more ranges than claimers the caller hands out
 // every further range through a counter (wants_claim / claimed), so that compute units that run
 // faster (the clocks of the eight XCDs differ by several per cent) take more of them.
+// Streamed sharing (split_dyn != 0; few shared tiles, short shares): the claimers are dealt out
+// over the shared tiles in contiguous groups (consecutive workgroups sit on different XCDs);
+// member g of a tile's group owns KV iterations [g s0, (g+1) s0) of the tile and then draws the
+// remaining iterations one at a time from the tile's counter, so that a group ends together
+// however its members' speeds differ.  Which iterations land in which partial result then
+// depends on timing: results are reproducible only to rounding.
 struct WorkgroupWalk {
   int whole_tile;  // a whole query tile still to do (< 0: none)
   int u_next;      // the range to take next (< 0: none)
@@ -77,7 +88,7 @@ struct WorkgroupWalk {
   template <typename P>
   XDIT_HD bool next(const P& p, int nt, Segment& s) {
     if (whole_tile >= 0) {
-      s.tile = whole_tile; s.it0 = 0; s.it1 = nt; s.slot = -1;
+      s.tile = whole_tile; s.it0 = 0; s.it1 = nt; s.slot = -1; s.dyn = -1; s.pool0 = 0;
       whole_tile = -1;
       return true;
     }
@@ -87,6 +98,24 @@ struct WorkgroupWalk {
       u_next = -1;
       lin = u * p.split_len;
       lin_end = lin + p.split_len < rem_iters ? lin + p.split_len : rem_iters;
+      if (p.split_dyn != 0) lin = lin_end = 0;
+    }
+    s.dyn = -1;
+    s.pool0 = 0;
+    if (p.split_dyn != 0) {  // one segment: this claimer's place in its tile's group
+      const int rem = p.total_tiles - p.split_full;
+      const int r = (int)(((int64_t)u * rem) / p.split_claimers);
+      const int c0 = (int)(((int64_t)r * p.split_claimers + rem - 1) / rem);
+      const int c1 = (int)(((int64_t)(r + 1) * p.split_claimers + rem - 1) / rem);
+      const int g = u - c0;
+      s.tile = p.split_full + r;
+      s.it0 = g * p.split_s0;
+      s.it1 = s.it0 + p.split_s0;
+      s.slot = (int64_t)r * p.split_pmax + g;
+      s.dyn = r;
+      s.pool0 = (c1 - c0) * p.split_s0;
+      lin = lin_end = 0;
+      return true;
     }
     const int r = lin / nt;  // which of the remaining query tiles
     s.it0 = lin - r * nt;
@@ -111,6 +140,10 @@ struct WorkgroupWalk {
 // workspace slots r * split_pmax + [0, parts).
 template <typename P>
 XDIT_HD int shared_tile_parts(const P& p, int nt, int r) {
+  if (p.split_dyn != 0) {
+    const int rem = p.total_tiles - p.split_full;
+    return (int)(((int64_t)(r + 1) * p.split_claimers + rem - 1) / rem) - (int)(((int64_t)r * p.split_claimers + rem - 1) / rem);
+  }
   const int first_unit = (r * nt) / p.split_len;
   const int last_unit = ((r + 1) * nt - 1) / p.split_len;
   return last_unit - first_unit + 1;

@@ -62,7 +62,11 @@ struct AttnParams {
   int split_fuse0;    // first workgroup that takes a range after its own query tile (> split_full: none)
   int split_share;    // KV iterations of the remaining query tiles per resident workgroup
   int split_claimers; // workgroups that process ranges
-  unsigned* split_counter;  // ranges handed out beyond the first of every claimer (nullptr: one range each)
+  unsigned* split_counter;  // ranges handed out beyond the first of every claimer (nullptr: one range each);
+                            // streamed sharing: one counter of KV iterations per shared tile
+  int split_dyn;      // streamed sharing of the remaining tiles (see WorkgroupWalk)
+  int split_s0;       // KV iterations every member of a tile's group owns before it draws from the counter
+  int deterministic;  // fixed work geometry only (no streamed sharing): results reproducible bit for bit
   // ring step (optional): the result is folded into an fp32 accumulator in the epilogue
   float* acc_out;     // (B,H,Sq,D) fp32 running output, nullptr: plain forward
   float* acc_lse;     // (B,H,Sq) fp32 running log-sum-exp
@@ -70,6 +74,8 @@ struct AttnParams {
   int64_t al_b, al_h, al_s;
   int acc_first;      // initialise the accumulator from this block instead of folding
   int acc_store;      // write acc_out back (0: only `out` and acc_lse receive the result)
+  unsigned* ws_counters;  // workspace: its counter region (start of the workspace)
+  int ws_preserved;   // the caller vouches that the counter region is as this library's last call left it
   void* ws_out;       // workspace: partial outputs [tile][slot][row][D] in the output dtype ...
   float* ws_lse;      // ... followed by partial log-sum-exps [tile][slot][row]
   size_t ws_bytes;

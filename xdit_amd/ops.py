@@ -62,23 +62,31 @@ class _on_device:
 
 
 _WORKSPACE = {}
+_RETIRED = []
 
 
 def _workspace(device, stream, nbytes):
-    """Per-device scratch tensor for balanced launches, grown on demand.  Calls on one stream are
-    ordered, so one buffer per (device, stream) can be reused from call to call."""
+    """Per-device scratch tensor for balanced launches, grown on demand -> (tensor, preserved).
+    Calls on one stream are ordered, so one buffer per (device, stream) is reused from call to
+    call; nothing else ever writes it, which is what `workspace_preserved` tells the library from
+    the second call on.  A buffer that has become too small is kept alive rather than freed, so
+    that its address cannot come back as a new buffer with foreign contents."""
     key = (device, stream)
-    buf = _WORKSPACE.get(key)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
-        _WORKSPACE[key] = buf
-    return buf
+    entry = _WORKSPACE.get(key)
+    if entry is None or entry[0].numel() < nbytes:
+        if entry is not None:
+            _RETIRED.append(entry[0])
+        entry = [torch.empty(int(nbytes), dtype=torch.uint8, device=device), 0]
+        _WORKSPACE[key] = entry
+    preserved = entry[1]   # 0 on a buffer's first use: its contents are arbitrary
+    entry[1] = 1
+    return entry[0], preserved
 
 
 # Launch tuning passed to the library with every attention call (fields of xdit_attn_args):
 # rows_per_workgroup 0 = the library's choice, else 128 / 256 / 384; cu_count 0 = the device's
 # compute units, else plan the launch as for that many.  Tests and sweeps set these.
-TUNING = {"rows_per_workgroup": 0, "cu_count": 0}
+TUNING = {"rows_per_workgroup": 0, "cu_count": 0, "deterministic": 0}
 
 # Argument structs are filled once per call signature (shapes, strides, dtypes, options) and kept:
 # a later call with the same signature only patches the pointers and the stream.
@@ -94,7 +102,7 @@ def _sig(t):
     return None if t is None else (t.shape, t.stride(), t.device)
 
 
-def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype, out, lse, acc):
+def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype, out, lse, acc, deterministic):
     device = q.device
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check4(name, t, device)
@@ -111,6 +119,7 @@ def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype
     a.B, a.H, a.D = B, H, D
     a.rows_per_workgroup = int(TUNING["rows_per_workgroup"])
     a.cu_count = int(TUNING["cu_count"])
+    a.deterministic = 1 if deterministic else 0
     a.Sq, a.Sk = Sq, k.shape[2]
     a.softmax_scale = float(softmax_scale)
     a.q_stride, a.k_stride, a.v_stride = _strides(q), _strides(k), _strides(v)
@@ -174,7 +183,7 @@ def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype
 
 def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
              q_descale=None, k_descale=None, v_descale=None, out_dtype=None, out=None,
-             return_lse=True, balance=True, lse=None, noalloc=False, _acc=None):
+             return_lse=True, balance=True, lse=None, noalloc=False, deterministic=None, _acc=None):
     """Non-causal attention forward on logical BHSD tensors -> (out BHSD, lse (B,H,Sq) fp32).
 
     `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
@@ -182,6 +191,9 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     `out` / `lse` receive the results when given (new tensors otherwise).
     `balance=False` withholds the scratch buffer with which the library evens out the last round
     of workgroups (results then come from one workgroup per query tile).
+    `deterministic=True` asks for results that are reproducible bit for bit from call to call; by
+    default (the reference passes deterministic=False everywhere) a balanced launch may share
+    the KV iterations of a query tile dynamically and results are reproducible to rounding.
     `noalloc=True` goes through the library's entry point that allocates nothing: the scratch is
     a fixed buffer inside the library (problems that need more than it holds raise ValueError),
     and `out` (and `lse` when `return_lse`) must be given.
@@ -199,14 +211,16 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
         raise ValueError("noalloc needs out (and lse) from the caller and is not available for the ring step")
     if lse is not None:
         return_lse = True
+    if deterministic is None:
+        deterministic = bool(TUNING["deterministic"])
     acc_sig = None if _acc is None else (_sig(_acc[0]), _sig(_acc[1]), _acc[2], _acc[3])
     key = (q.dtype, out_dtype, device, _sig(q), _sig(k), _sig(v), _sig(k2), _sig(v2), _sig(out), _sig(lse),
            k.dtype, v.dtype, float(softmax_scale), bool(causal), q_descale is not None, k_descale is not None,
-           v_descale is not None, acc_sig, TUNING["rows_per_workgroup"], TUNING["cu_count"])
+           v_descale is not None, acc_sig, TUNING["rows_per_workgroup"], TUNING["cu_count"], bool(deterministic))
     plan = _PLANS.get(key)
     if plan is None:
         plan = _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, (q_descale, k_descale, v_descale),
-                                out_dtype, out, lse, _acc)
+                                out_dtype, out, lse, _acc, deterministic)
         if len(_PLANS) >= _PLANS_MAX:
             _PLANS.clear()
         _PLANS[key] = plan
@@ -241,17 +255,17 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
             rc = L.xdit_attn_fwd_noalloc(ctypes.byref(a))
         else:
             if balance and plan.need > 0:
-                ws = _workspace(device, stream, plan.need)
-                a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+                ws, preserved = _workspace(device, stream, plan.need)
+                a.workspace, a.workspace_bytes, a.workspace_preserved = ws.data_ptr(), ws.numel(), preserved
             else:
-                a.workspace, a.workspace_bytes = None, 0
+                a.workspace, a.workspace_bytes, a.workspace_preserved = None, 0, 0
             rc = L.xdit_attn_fwd(ctypes.byref(a))
     if rc != 0:
         _lib.check(rc)
     return out, lse
 
 
-def launch_plan(q, k, k2=None):
+def launch_plan(q, k, k2=None, deterministic=None):
     """How `attn_fwd(q, k, v, k2=..)` would be launched (a dict of the fields of xdit_launch_plan):
     rows per workgroup, query tiles, whole tiles, shared ranges and their length, claimers,
     whether ranges are handed out through the counter, workgroups, workspace bytes.  Host
@@ -265,6 +279,7 @@ def launch_plan(q, k, k2=None):
     a.Sk2 = 0 if k2 is None else k2.shape[2]
     a.rows_per_workgroup = int(TUNING["rows_per_workgroup"])
     a.cu_count = int(TUNING["cu_count"])
+    a.deterministic = 1 if (TUNING["deterministic"] if deterministic is None else deterministic) else 0
     p = _lib.LaunchPlan()
     p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
     _lib.check(_lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)))
