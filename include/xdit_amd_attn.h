@@ -184,7 +184,8 @@ int xdit_attn_launch_plan(const xdit_attn_args* args, xdit_launch_plan* plan);
  * If final_out != NULL the merged row is also written there in final_dtype (the epilogue cast
  * `out.to(q.dtype)`).  acc_out/block_out/final_out are logical (B,H,S,D); acc_lse/block_lse are
  * logical (B,H,S) with their own B/H/S strides, so the (B,S,H,1) accumulator layout of the legacy
- * ring and the (B,H,S) layout a kernel returns both map without copies.
+ * ring and the (B,H,S) layout a kernel returns both map without copies.  head_dim: a multiple of
+ * 8 up to 512.
  * Replaces: update_out_and_lse at ring_flash_attn.py:138, the epilogue at :145, and
  * torch _SDPAMerger._merge_one (…/_context_parallel/_attention.py:161-163, :181-182).
  */
@@ -246,7 +247,14 @@ int xdit_attn_fwd_accumulate(const xdit_attn_args* args, const xdit_ring_acc* ac
  * `scale.expand(B, H)`.  `per_tensor == 0`: one abs-max per (batch, head) slice.
  * `scale_in != NULL` (device pointer to one float) supplies a static scale instead of the abs-max
  * (the `scale=` argument of per_tensor_quant).  Values whose quotient exceeds 448 saturate.
- * `descale` (B*H contiguous fp32) doubles as the reduction buffer; no other memory is used.
+ * `x2` / `y2` (S2 > 0): a second tensor (B,H,S2,D) quantised with the scales of the first, the
+ * abs-max taken over both (the joint keys, or values, that a caller would otherwise torch.cat onto
+ * the first tensor before quantising: usp.py:239-241 in front of attention_backend.py:606-615).
+ * `scratch`: optional device memory of at least XDIT_FP8_QUANT_SCRATCH_BYTES(B, H) bytes, private
+ * to the stream until the call's kernels finish, no initialisation needed.  With it the call is
+ * two launches (abs-max with one scratch slot per workgroup; cast), one with a static scale.
+ * Without it `descale` (B*H contiguous fp32) doubles as the reduction buffer and the call is four
+ * launches (clear, abs-max through atomics, cast, descales); results are the same.
  * `hadamard_block` (0 or 1 = off; else a power of two <= 128 that divides D) first rotates every
  * row along head_dim, block by block, by the orthonormal Sylvester-Hadamard matrix R of that size
  * with entries +-r, r = 1/sqrt(block) rounded to in_dtype, and rounds the result to in_dtype:
@@ -268,7 +276,15 @@ typedef struct {
   void* stream;
   int32_t hadamard_block;
   int32_t reserved0;
+  int64_t S2;                  /* rows of the second tensor (0 = none) */
+  const void* x2;              /* (B,H,S2,D) in_dtype */
+  void* y2;                    /* (B,H,S2,D) fp8 e4m3fn bytes */
+  xdit_strides x2_stride, y2_stride;
+  void* scratch;               /* optional, may be NULL */
+  int64_t scratch_bytes;
 } xdit_quant_args;
+
+#define XDIT_FP8_QUANT_SCRATCH_BYTES(B, H) (4 * ((int64_t)(B) * (H) > 4096 ? (int64_t)(B) * (H) : 4096))
 
 int xdit_fp8_quant(const xdit_quant_args* args);
 

@@ -455,7 +455,7 @@ def test_merge_vs_oracle(gpu, block_dtype, layout):
     assert torch.equal(fo, ao.bfloat16())
 
 
-@pytest.mark.parametrize("D", [72, 40, 104, 520])
+@pytest.mark.parametrize("D", [72, 40, 104, 512])
 def test_merge_rows_that_do_not_fill_a_wavefront(gpu, D):
     """head_dim / 8 that does not divide 64 (72 is PixArt's, the head_dim of the fp32 ring): with a
     flat thread -> chunk map a row straddles two wavefronts or workgroups and its later lanes can
@@ -802,6 +802,88 @@ def test_fp8_backend_adapter(gpu):
     o, l = AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355_FP8](q.to(gpu), k.to(gpu), v.to(gpu), 0.0, False)
     assert o.dtype == torch.bfloat16 and _err(o, ro) <= 6e-2 and _err(l, rl) <= 5e-2  # vs the UNQUANTISED inputs
     assert torch.equal(o, usp.attention(q.to(gpu), k.to(gpu), v.to(gpu), backend=AB.AttentionBackendType.MI355_FP8))
+
+
+@pytest.mark.parametrize("strategy", ["rear", "front"])
+def test_fp8_backend_adapter_joint_keys_without_a_copy(gpu, monkeypatch, strategy):
+    """The fp8 adapter with joint (text) keys/values: they are quantised with the scale of the
+    keys/values they are attended with (one abs-max over both) and handed to the kernel as its
+    second KV segment.  Bytes and scales must equal what quantising the concatenation gives (the
+    reference's order of operations: usp.py:239-241, then per_tensor_quant), no torch.cat of K or
+    V may run, and the output must match the oracle's attention of the dequantised tensors."""
+    q, k, v = O.make_qkv(1, 3, 400, 128, seed=71, dtype=torch.bfloat16)
+    _, jk, jv = O.make_qkv(1, 3, 77, 128, seed=72, dtype=torch.bfloat16)
+    jk = jk * 1.5  # the joint keys carry the abs-max
+    order = (lambda a, b: torch.cat([a, b], 2)) if strategy == "rear" else (lambda a, b: torch.cat([b, a], 2))
+    k8, j8, kd = AB.per_tensor_quant(k.to(gpu), x2=jk.to(gpu))
+    rk8, rkd = O.per_tensor_quant_ref(torch.cat([k, jk], 2))
+    assert torch.equal(torch.cat([k8, j8], 2).cpu().view(torch.uint8), rk8.view(torch.uint8)) and torch.equal(kd.cpu(), rkd.contiguous())
+    # reference of the whole call: quantise q, cat(k), cat(v) per tensor, attend the dequantised tensors
+    (q8, qd), (kk8, kkd), (vv8, vvd) = (O.per_tensor_quant_ref(t) for t in (q, order(k, jk), order(v, jv)))
+    ro, rl = O.attn_fwd_ref(O.dequant(q8, qd), O.dequant(kk8, kkd), O.dequant(vv8, vvd))
+    cats = []
+    real_cat = torch.cat
+    monkeypatch.setattr(torch, "cat", lambda *a, **kw: (cats.append(1), real_cat(*a, **kw))[1])
+    fn = AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355_FP8]
+    o, l = fn(q.to(gpu), k.to(gpu), v.to(gpu), 0.0, False, attention_kwargs={"hadamard_block": 0},
+              joint_kv=(jk.to(gpu), jv.to(gpu), strategy))
+    monkeypatch.undo()
+    assert not cats
+    # (keys wider than unit RMS concentrate the softmax on few keys, the hard case for an fp8 P:
+    # the bar is applied relative to the largest output where that exceeds 1)
+    assert _err(o, ro) <= 6e-2 * max(1.0, ro.abs().max().item()) and _err(l, rl) <= 1e-3
+    # through USP, with the rotation on (the default): the same call as the adapter's, and close to
+    # the attention of the unquantised tensors (which also sees the fp8 rounding of q, k and v)
+    uo = usp.USP(q[:, :, :300].to(gpu), k.to(gpu), v.to(gpu), joint_query=q[:, :, 300:].to(gpu), joint_key=jk.to(gpu),
+                 joint_value=jv.to(gpu), joint_strategy=strategy, backend=AB.AttentionBackendType.MI355_FP8)
+    qq = order(q[:, :, :300], q[:, :, 300:])
+    direct, _ = fn(qq.to(gpu), k.to(gpu), v.to(gpu), 0.0, False, joint_kv=(jk.to(gpu), jv.to(gpu), strategy))
+    assert torch.equal(uo, direct)
+    fo, _ = O.attn_fwd_ref(qq, order(k, jk), order(v, jv))
+    assert _err(uo, fo) <= 0.25
+
+
+def test_fp8_backend_adapter_static_scale(gpu, monkeypatch):
+    """A static scale for q, k and v (the reference takes one from
+    XFUSER_AITER_FP8_STATIC_SCALE_WITH_DESCALE, attention_backend.py:735-745): per call through
+    attention_kwargs or as the module's default; descales then equal the scale."""
+    q, k, v = O.make_qkv(1, 2, 256, 128, seed=81, dtype=torch.bfloat16)
+    s = 0.02
+    (q8, qd), (k8, kd), (v8, vd) = (O.per_tensor_quant_ref(t.clamp(-448 * s, 448 * s), scale=torch.tensor(s)) for t in (q, k, v))
+    ro, rl = O.attn_fwd_ref(O.dequant(q8, qd), O.dequant(k8, kd), O.dequant(v8, vd))
+    fn = AB.ATTENTION_FUNCTION_REGISTRY[AB.AttentionBackendType.MI355_FP8]
+    o, l = fn(q.to(gpu), k.to(gpu), v.to(gpu), 0.0, False, attention_kwargs={"hadamard_block": 0, "fp8_static_scale": s})
+    assert _err(o, ro) <= 6e-2 and _err(l, rl) <= 1e-3
+    monkeypatch.setattr(AB, "FP8_STATIC_SCALE", s)
+    o2, l2 = fn(q.to(gpu), k.to(gpu), v.to(gpu), 0.0, False, attention_kwargs={"hadamard_block": 0})
+    assert torch.equal(o, o2) and torch.equal(l, l2)
+
+
+def test_fp8_quant_with_and_without_scratch(gpu):
+    """The quantiser through the C ABI with no scratch buffer (four launches, atomics on the descale
+    buffer) and with one (two launches): the same bytes and descales, per head and per tensor, with
+    a second tensor sharing the scales."""
+    import ctypes
+    from xdit_amd import _lib
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(2, 3, 301, 128, generator=g) * torch.arange(1, 7).reshape(2, 3, 1, 1)).bfloat16().to(gpu)
+    x2 = (torch.randn(2, 3, 40, 128, generator=g) * 9).bfloat16().to(gpu)
+    for per_tensor in (False, True):
+        want = ops.fp8_quant(x, per_tensor=per_tensor, x2=x2)
+        ry, rd = (O.per_tensor_quant_ref if per_tensor else O.per_head_quant_ref)(torch.cat([x, x2], 2).cpu())
+        assert torch.equal(torch.cat(want[:2], 2).cpu().view(torch.uint8), ry.view(torch.uint8)) and torch.equal(want[2].cpu(), rd.contiguous())
+        y = torch.empty_like(want[0]); y2 = torch.empty_like(want[1]); d = torch.empty_like(want[2])
+        a = _lib.QuantArgs()
+        a.struct_size = ctypes.sizeof(_lib.QuantArgs)
+        a.in_dtype, a.per_tensor = _lib.DTYPE_BF16, int(per_tensor)
+        a.B, a.H, a.D, a.S, a.S2 = 2, 3, 128, 301, 40
+        a.x, a.y, a.descale, a.x2, a.y2 = x.data_ptr(), y.data_ptr(), d.data_ptr(), x2.data_ptr(), y2.data_ptr()
+        a.x_stride, a.y_stride = ops._strides(x), ops._strides(y)
+        a.x2_stride, a.y2_stride = ops._strides(x2), ops._strides(y2)
+        a.stream = ops._stream(x.device)
+        _lib.check(_lib.lib().xdit_fp8_quant(ctypes.byref(a)))   # scratch = NULL
+        torch.cuda.synchronize()
+        assert all(torch.equal(p.view(torch.uint8), r.view(torch.uint8)) for p, r in ((y, want[0]), (y2, want[1]))) and torch.equal(d, want[2])
 
 
 def test_runs_on_the_callers_stream(gpu):

@@ -142,6 +142,13 @@ class QuantArgs(ctypes.Structure):
         ("stream", ctypes.c_void_p),
         ("hadamard_block", ctypes.c_int32),
         ("reserved0", ctypes.c_int32),
+        ("S2", ctypes.c_int64),
+        ("x2", ctypes.c_void_p),
+        ("y2", ctypes.c_void_p),
+        ("x2_stride", Strides),
+        ("y2_stride", Strides),
+        ("scratch", ctypes.c_void_p),
+        ("scratch_bytes", ctypes.c_int64),
     ]
 
 

@@ -7,6 +7,7 @@ on BHSD tensors (:504-516 for the prototype, :774-823 for what HIP devices run t
 The two adapters here call the gfx950 kernels through the C ABI.  Unlike the reference's AITER
 adapter (:780-782) nothing is permuted or made contiguous: the kernels take BHSD strides.
 """
+import os
 from enum import Enum
 
 import torch
@@ -90,28 +91,37 @@ def get_dtype_max(dtype):
 FP8_HADAMARD_BLOCK = 128
 
 
+# Static scale of the fp8 adapter for q, k and v alike, as the reference's AITER fp8 adapter takes
+# one from XFUSER_AITER_FP8_STATIC_SCALE_WITH_DESCALE (attention_backend.py:735-745); None = dynamic
+# (abs-max) scaling.  attention_kwargs["fp8_static_scale"] overrides it per call.
+_env_scale = os.environ.get("XFUSER_AITER_FP8_STATIC_SCALE_WITH_DESCALE")
+FP8_STATIC_SCALE = float(_env_scale) if _env_scale not in (None, "") else None
+
+
 def per_tensor_quant(x, scale=None, scale_dtype=torch.float32, quant_dtype=torch.float8_e4m3fn, dtypeMax=None,
-                     hadamard_block=0):
+                     hadamard_block=0, x2=None):
     """Same contract as the reference's per_tensor_quant (attention_backend.py:606-615):
     one abs-max scale over the whole tensor, y = fp8(x / scale), descale expanded to x.shape[:2].
     With `scale=None` the abs-max reduction and the cast run in the HIP quantiser.
     `hadamard_block` fuses _fp8_hadamard_rotate (:703-714) in front: x is rotated along head_dim
-    in blocks of that size before the abs-max and the cast."""
+    in blocks of that size before the abs-max and the cast.  `x2` (the joint keys or values) is
+    quantised with the same scale, the abs-max taken over both tensors as if they had been
+    concatenated first; the result is then (y, y2, descale)."""
     if quant_dtype != torch.float8_e4m3fn:
         raise NotImplementedError("only float8_e4m3fn (the fp8 format of gfx950) is supported")
     if scale is None and dtypeMax in (None, get_dtype_max(quant_dtype)):
-        if torch.compiler.is_compiling():
+        if torch.compiler.is_compiling() and x2 is None:
             y, descale = torch.ops.xdit_amd.fp8_quant(x, True, hadamard_block)
-        else:
-            y, descale = ops.fp8_quant(x, per_tensor=True, hadamard_block=hadamard_block)
-        return y, descale.to(scale_dtype)
+            return y, descale.to(scale_dtype)
+        out = ops.fp8_quant(x, per_tensor=True, hadamard_block=hadamard_block, x2=x2)
+        return (*out[:-1], out[-1].to(scale_dtype))
     if scale is None:
-        if hadamard_block > 1:
-            raise NotImplementedError("a non-default dtypeMax together with the fused rotation is not implemented")
+        if hadamard_block > 1 or x2 is not None:
+            raise NotImplementedError("a non-default dtypeMax together with the fused rotation or a second tensor is not implemented")
         scale = torch.abs(x.to(torch.float32)).max() / dtypeMax
     scale = torch.as_tensor(scale, dtype=torch.float32, device=x.device)
-    y, descale = ops.fp8_quant(x, per_tensor=True, scale=scale, hadamard_block=hadamard_block)
-    return y, descale.to(scale_dtype)
+    out = ops.fp8_quant(x, per_tensor=True, scale=scale, hadamard_block=hadamard_block, x2=x2)
+    return (*out[:-1], out[-1].to(scale_dtype))
 
 
 @register_attention_function(AttentionBackendType.MI355_FP8)
@@ -124,23 +134,38 @@ def _mi355_fp8_attn_call(query, key, value, dropout_p, is_causal, attention_kwar
     Inputs that are already float8_e4m3fn take their descales from attention_kwargs
     ("q_descale", "k_descale", "v_descale")."""
     _check_call(dropout_p, is_causal, attention_kwargs)
-    if joint_kv is not None:
-        key = torch.cat([key, joint_kv[0]] if joint_kv[2] == "rear" else [joint_kv[0], key], dim=2)
-        value = torch.cat([value, joint_kv[1]] if joint_kv[2] == "rear" else [joint_kv[1], value], dim=2)
+    kw = attention_kwargs or {}
     scale = query.shape[-1] ** -0.5
+    jk = jv = strategy = None
+    if joint_kv is not None:
+        jk, jv, strategy = joint_kv
+        if strategy not in ("front", "rear"):
+            raise ValueError(f"Invalid joint_strategy: {strategy}")
     if query.dtype == torch.float8_e4m3fn:
-        kw = attention_kwargs or {}
-        return ops.attn_fwd(query, key, value, softmax_scale=scale, q_descale=kw.get("q_descale"),
+        k1, v1, k2, v2 = _split_joint(key, value, joint_kv)
+        return ops.attn_fwd(query, k1, v1, softmax_scale=scale, k2=k2, v2=v2, q_descale=kw.get("q_descale"),
                             k_descale=kw.get("k_descale"), v_descale=kw.get("v_descale"),
                             out_dtype=kw.get("out_dtype", torch.bfloat16))
     out_dtype = query.dtype if query.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
-    had = (attention_kwargs or {}).get("hadamard_block", FP8_HADAMARD_BLOCK)
+    had = kw.get("hadamard_block", FP8_HADAMARD_BLOCK)
     if had > 1 and query.shape[-1] % had != 0:
         had = 0
+    static = kw.get("fp8_static_scale", FP8_STATIC_SCALE)
     # rotating q and k alike leaves q.k unchanged and spreads outliers before the fp8 cast
-    q8, qd = per_tensor_quant(query, hadamard_block=had)
-    k8, kd = per_tensor_quant(key, hadamard_block=had)
-    v8, vd = per_tensor_quant(value)
-    if torch.compiler.is_compiling():
+    q8, qd = per_tensor_quant(query, scale=static, hadamard_block=had)
+    if jk is None:
+        k8, kd = per_tensor_quant(key, scale=static, hadamard_block=had)
+        v8, vd = per_tensor_quant(value, scale=static)
+        k2 = v2 = None
+    else:
+        # the joint keys / values share the scale of the keys / values they are attended with (one
+        # abs-max over both, as quantising their concatenation would give) and go to the kernel as
+        # its second KV segment: no concatenated copy of K and V is made
+        k8, k2, kd = per_tensor_quant(key, scale=static, hadamard_block=had, x2=jk)
+        v8, v2, vd = per_tensor_quant(value, scale=static, x2=jv)
+        if strategy == "front":
+            k8, v8, k2, v2 = k2, v2, k8, v8
+    if torch.compiler.is_compiling() and k2 is None:
         return torch.ops.xdit_amd.attn_fwd_fp8(q8, k8, v8, qd, kd, vd, scale, out_dtype == torch.float16)
-    return ops.attn_fwd(q8, k8, v8, softmax_scale=scale, q_descale=qd, k_descale=kd, v_descale=vd, out_dtype=out_dtype)
+    return ops.attn_fwd(q8, k8, v8, softmax_scale=scale, k2=k2, v2=v2, q_descale=qd, k_descale=kd, v_descale=vd,
+                        out_dtype=out_dtype)

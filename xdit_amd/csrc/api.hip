@@ -394,7 +394,7 @@ int xdit_lse_merge(const xdit_merge_args* a) {
   if (a->block_dtype != XDIT_DTYPE_BF16 && a->block_dtype != XDIT_DTYPE_FP16 && a->block_dtype != XDIT_DTYPE_FP32)
     return fail(XDIT_ERR_INVALID_ARG, "block_dtype %d must be bf16, fp16 or fp32", a->block_dtype);
   if (a->B <= 0 || a->H <= 0 || a->S <= 0) return fail(XDIT_ERR_INVALID_ARG, "B, H, S must be positive");
-  if (a->D <= 0 || a->D % 8 != 0) return fail(XDIT_ERR_INVALID_ARG, "head_dim %d must be a positive multiple of 8", a->D);
+  if (a->D <= 0 || a->D % 8 != 0 || a->D > 512) return fail(XDIT_ERR_INVALID_ARG, "head_dim %d must be a positive multiple of 8, at most 512", a->D);
   if (a->S > (int64_t(1) << 30)) return fail(XDIT_ERR_INVALID_ARG, "S above 2^30");
   if (a->acc_lse == nullptr || a->block_lse == nullptr) return fail(XDIT_ERR_INVALID_ARG, "acc_lse / block_lse is NULL");
   int rc;
@@ -443,6 +443,14 @@ int xdit_fp8_quant(const xdit_quant_args* a) {
   if ((reinterpret_cast<uintptr_t>(a->y) & 7u) || a->y_stride.b % 8 || a->y_stride.h % 8 || a->y_stride.s % 8)
     return fail(XDIT_ERR_INVALID_ARG, "y must be 8-byte aligned with strides that are multiples of 8");
   if (a->y_stride.s < a->D) return fail(XDIT_ERR_INVALID_ARG, "y: S stride smaller than head_dim");
+  if (a->S2 < 0 || a->S2 > (int64_t(1) << 30)) return fail(XDIT_ERR_INVALID_ARG, "S2 must be between 0 and 2^30");
+  if (a->S2 > 0) {
+    if ((rc = check_tensor("x2", a->x2, a->x2_stride, elem_size(a->in_dtype), a->D))) return rc;
+    if (a->y2 == nullptr) return fail(XDIT_ERR_INVALID_ARG, "y2 is NULL");
+    if ((reinterpret_cast<uintptr_t>(a->y2) & 7u) || a->y2_stride.b % 8 || a->y2_stride.h % 8 || a->y2_stride.s % 8)
+      return fail(XDIT_ERR_INVALID_ARG, "y2 must be 8-byte aligned with strides that are multiples of 8");
+    if (a->y2_stride.s < a->D) return fail(XDIT_ERR_INVALID_ARG, "y2: S stride smaller than head_dim");
+  }
   const int hb = a->hadamard_block;
   if (hb < 0 || hb > 128 || (hb & (hb - 1)) != 0 || (hb > 1 && a->D % hb != 0))
     return fail(XDIT_ERR_INVALID_ARG, "hadamard_block %d must be 0 or a power of two <= 128 that divides head_dim %d", hb, a->D);
@@ -455,6 +463,19 @@ int xdit_fp8_quant(const xdit_quant_args* a) {
   p.ys_b = a->y_stride.b; p.ys_h = a->y_stride.h; p.ys_s = a->y_stride.s;
   p.B = a->B; p.H = a->H; p.S = (int)a->S; p.D = a->D;
   p.per_tensor = a->per_tensor ? 1 : 0;
+  if (a->S2 > 0) {
+    p.x2 = a->x2; p.y2 = a->y2; p.S2 = (int)a->S2;
+    p.x2s_b = a->x2_stride.b; p.x2s_h = a->x2_stride.h; p.x2s_s = a->x2_stride.s;
+    p.y2s_b = a->y2_stride.b; p.y2s_h = a->y2_stride.h; p.y2s_s = a->y2_stride.s;
+  }
+  if (a->scratch != nullptr && (reinterpret_cast<uintptr_t>(a->scratch) & 3u) == 0 &&
+      a->scratch_bytes >= XDIT_FP8_QUANT_SCRATCH_BYTES(a->B, a->H)) {
+    p.partials = (float*)a->scratch;
+    p.partial_slots = a->scratch_bytes / 4;
+    if (p.partial_slots > 65536) p.partial_slots = 65536;
+    const int64_t bh = (int64_t)a->B * a->H;
+    if (p.partial_slots < bh) p.partials = nullptr;
+  }
   hipError_t e = xdit::launch_fp8_quant(p, a->in_dtype, (hipStream_t)a->stream);
   if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "quantiser launch failed: %s", hipGetErrorString(e));
   return XDIT_OK;

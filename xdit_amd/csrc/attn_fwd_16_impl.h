@@ -68,34 +68,6 @@ constexpr int lds_bytes_16() {
 // not stored.  DC (a multiple of 16, d_actual <= DC <= D) is the head_dim the two products are
 // computed over: LDS tiles keep the geometry of D, contraction steps (of 16) and output blocks
 // (of 32) past DC are left out.
-// The lane's index within its wavefront, computed where it is called (two instructions) instead
-// of being kept in a register through the KV loop; not merged with other calls by the compiler.
-__device__ __forceinline__ int lane_now() {
-  int x;
-  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(x));
-  return x;
-}
-
-// One ticket from a counter in device memory (device-scope atomic add of 1, relaxed), for a branch
-// that a single lane takes.  The operands are formed right here rather than kept in registers
-// through the KV loop around it.
-__device__ __forceinline__ unsigned draw_ticket(unsigned* counter) {
-  unsigned one = 1;
-  asm volatile("" : "+v"(one));
-  return __hip_atomic_fetch_add(counter, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// The launch geometry the walker reads, gathered from the kernel arguments when needed.
-struct WalkGeom {
-  int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers, split_dyn, split_s0;
-};
-typedef const __attribute__((address_space(4))) AttnParams* ParamsPtr;
-__device__ __forceinline__ WalkGeom walk_geom(ParamsPtr pp) {
-  WalkGeom g = {pp->total_tiles, pp->tiles_per_xcd, pp->split_full, pp->split_units, pp->split_len, pp->split_pmax,
-                pp->split_fuse0, pp->split_claimers, pp->split_dyn, pp->split_s0};
-  return g;
-}
-
 // The kernel's only argument is read in place, through a pointer to the kernel-argument segment
 // that is made opaque to the compiler after every KV loop: what a segment's prologue and
 // epilogue need is then loaded (scalar loads) when it is needed instead of being kept in

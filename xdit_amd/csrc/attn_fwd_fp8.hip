@@ -41,281 +41,359 @@ constexpr int BUF_BYTES = K_BYTES + V_BYTES;
 // LDS fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
 constexpr int kPrefetch = 2;
 
-// One segment of work: query tile `tile`, KV tiles [it0, it1); see attn_split.h for part_out.
+// Output staging block of a wavefront in the epilogue: 32 rows of 64 16-bit columns, rows 8 bytes
+// apart from a multiple of 128 so that the 8-byte writes of the 32 lanes of a half hit 32 banks.
+constexpr int kStagePitch = 64 * 2 + 8;
+constexpr int kStageBytes = kRowsPerWave * kStagePitch;
+// LDS of a workgroup: the first K/V buffer, then a region that holds the second K/V buffer during
+// the KV loop and the output staging blocks of the wavefronts in the epilogue.
+template <int NW>
+constexpr int lds_bytes() { return BUF_BYTES + (BUF_BYTES > NW * kStageBytes ? BUF_BYTES : NW * kStageBytes); }
+
+// The work of one workgroup: its segments (WorkgroupWalk), one after the other; a segment is the
+// query tile `tile` and KV tiles [it0, it1), written to the output tensors (slot < 0) or as one
+// part of a shared query tile to its workspace slot.  As in the 16-bit kernel the kernel
+// arguments are read in place (and afresh after every KV loop, so that the loop keeps the
+// registers), the Q fragments and the first K/V tile of a workgroup's next segment are requested
+// ahead of the epilogue of the current one, and the rows leave through an LDS transpose as
+// whole 128-byte lines.
 template <typename TO, int NW>
-__device__ __forceinline__ void attn_segment_fp8(const AttnParams& p, unsigned char* smem, const int tile,
-                                                 const int it0, const int it1, TO* part_out, float* part_lse) {
+__device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
   typedef unsigned char u8;
+  ParamsPtr pp = (ParamsPtr)__builtin_amdgcn_kernarg_segment_ptr();
   constexpr int kWaves = NW;
   constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nt1 = (pp->Sk + kKeysPerTile - 1) / kKeysPerTile;
+  const int nt = nt1 + (pp->Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+  __shared__ unsigned ticket;
+  WorkgroupWalk walk;
+  Segment seg;
+  {
+    const WalkGeom g = walk_geom(pp);
+    if (!walk.start(g, nt, (int)blockIdx.x) || !walk.next(g, nt, seg)) return;
+  }
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int lane = lane_now();   // for the set-up below; later code asks again
   const int l32 = lane & 31;
   const int hh = lane >> 5;
 
-  const int bh = tile / p.nq_tiles;
-  const int qt = tile - bh * p.nq_tiles;
-  const int b = bh / p.H;
-  const int h = bh - b * p.H;
-
-  // ---- Q fragments: 2 contraction steps x 32 bytes ---------------------------------------
-  const int qrow = qt * kRowsPerBlock + wave * kRowsPerWave + l32;
-  const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
-  const u8* qptr = (const u8*)p.q + b * p.qs_b + h * p.qs_h + (int64_t)qrow_c * p.qs_s + hh * 32;
-  i32x8 qf[2];
-#pragma unroll
-  for (int ks = 0; ks < 2; ks++) {
-    i32x4 lo = *(const i32x4*)(qptr + ks * 64);
-    i32x4 hi = *(const i32x4*)(qptr + ks * 64 + 16);
-    qf[ks] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  }
-
   // ---- tile loads ------------------------------------------------------------------------
-  const u8* kbase1 = (const u8*)p.k + b * p.ks_b + h * p.ks_h;
-  const u8* vbase1 = (const u8*)p.v + b * p.vs_b + h * p.vs_h;
-  const u8* kbase2 = p.Sk2 > 0 ? (const u8*)p.k2 + b * p.k2s_b + h * p.k2s_h : kbase1;
-  const u8* vbase2 = p.Sk2 > 0 ? (const u8*)p.v2 + b * p.v2s_b + h * p.v2s_h : vbase1;
   // Loader wavefronts: the first LW wavefronts each load PAIRS (K piece g, V piece g) pairs,
   // g = wave + LW * i, with one row index per lane for both pieces of a pair.
   constexpr int LW = kWaves < 8 ? kWaves : 8;
   constexpr int PAIRS = NG / LW;
-  const int ld_row0 = NG * (lane >> 3) + wave;    // 8 lanes per 128-byte row: row of this lane in pair 0
-  const unsigned ld_colb = (lane & 7) * 16;
+  int ld_row0 = NG * (lane >> 3) + wave;    // 8 lanes per 128-byte row: row of this lane in pair 0
+  unsigned ld_colb = (lane & 7) * 16;
+  asm volatile("" : "+v"(ld_row0), "+v"(ld_colb));
   const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS u8*)smem;
   const unsigned ld_kdst = lds_base + wave * K_PITCH;  // LDS address of K piece `wave`, buffer 0
   const unsigned ld_vdst = lds_base + K_BYTES + wave * V_PITCH;
-  const int nt1 = (p.Sk + kKeysPerTile - 1) / kKeysPerTile;
 
-  // Stream position: base pointers of the next tile to load, byte strides, keys left in its segment.
-  const u8* ld_kp;
-  const u8* ld_vp;
-  unsigned ld_kss, ld_vss;
-  int64_t ld_kstep, ld_vstep;
-  int ld_left;
-  auto seek_tile = [&](int t) {
-    if (t < nt1) {
-      ld_kp = kbase1 + (int64_t)t * kKeysPerTile * p.ks_s;
-      ld_vp = vbase1 + (int64_t)t * kKeysPerTile * p.vs_s;
-      ld_kss = (unsigned)p.ks_s; ld_vss = (unsigned)p.vs_s;
-      ld_kstep = kKeysPerTile * p.ks_s; ld_vstep = kKeysPerTile * p.vs_s;
-      ld_left = p.Sk - t * kKeysPerTile;
-    } else {
-      ld_kp = kbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.k2s_s;
-      ld_vp = vbase2 + (int64_t)(t - nt1) * kKeysPerTile * p.v2s_s;
-      ld_kss = (unsigned)p.k2s_s; ld_vss = (unsigned)p.v2s_s;
-      ld_kstep = kKeysPerTile * p.k2s_s; ld_vstep = kKeysPerTile * p.v2s_s;
-      ld_left = p.Sk2 - (t - nt1) * kKeysPerTile;
-    }
-  };
-  // Loads the tile at the stream position into buffer `buf` and advances the position.
+  // Where the K/V rows of the current (batch, head) lie, set per segment (row strides in bytes).
+  const u8* kv_k1;
+  const u8* kv_v1;
+  const u8* kv_k2;
+  const u8* kv_v2;
+  unsigned kss1, vss1, kss2, vss2;
+  int keys1, keys2;
   auto issue_tile = [&](int t, int buf) {
     if (kWaves == LW || wave < LW) {
-      const int last = (ld_left < kKeysPerTile ? ld_left : kKeysPerTile) - 1;
+      const bool second = t >= nt1;
+      const unsigned row0 = (unsigned)(second ? t - nt1 : t) * kKeysPerTile;
+      const unsigned kss = second ? kss2 : kss1, vss = second ? vss2 : vss1;
+      const u8* kp = (second ? kv_k2 : kv_k1) + (uint64_t)row0 * kss;
+      const u8* vp = (second ? kv_v2 : kv_v1) + (uint64_t)row0 * vss;
+      const int left = (second ? keys2 : keys1) - (int)row0;
+      const int last = (left < kKeysPerTile ? left : kKeysPerTile) - 1;
       const unsigned bo = buf * BUF_BYTES;
 #pragma unroll
       for (int i = 0; i < PAIRS; i++) {
         int r = ld_row0 + LW * i;
         r = r < last ? r : last;  // rows past the end of the segment re-read its last row
-        load_lds_16(ld_kp, __umul24((unsigned)r, ld_kss) + ld_colb, ld_kdst + bo + i * LW * K_PITCH);
-        load_lds_16(ld_vp, __umul24((unsigned)r, ld_vss) + ld_colb, ld_vdst + bo + i * LW * V_PITCH);
+        load_lds_16(kp, __umul24((unsigned)r, kss) + ld_colb, ld_kdst + bo + i * LW * K_PITCH);
+        load_lds_16(vp, __umul24((unsigned)r, vss) + ld_colb, ld_vdst + bo + i * LW * V_PITCH);
       }
-    }
-    if (t + 1 == nt1) {
-      seek_tile(t + 1);
-    } else {
-      ld_kp += ld_kstep; ld_vp += ld_vstep; ld_left -= kKeysPerTile;
     }
   };
 
   // ---- LDS read bases ------------------------------------------------------------------------
   // K fragment for key block kb, step ks: row 32kb + l32, bytes 64ks + 32hh .. +31.
-  const int kbase_off = (l32 & 7) * K_PITCH + (l32 >> 3) * ROW_BYTES + hh * 32;
+  unsigned kbase_off = lds_base + (l32 & 7) * K_PITCH + (l32 >> 3) * ROW_BYTES + hh * 32;
   // V^T fragment, read r (0..3), d block db: as a SOURCE lane of ds_read_b64_tr_b8, lane
   // (group g = lane/16, s = lane%16) supplies 8 bytes of key row 16r + 8(s/8) + 4hh + (s/2)%4
   // at d = 32db + 16(g%2) + 8(s%2); lane (g, i) receives d = 32db + 16(g%2) + i for the 8 keys
   // 16r + 8(j/4) + 4hh + j%4, j = 0..7.
   const int s16 = lane & 15;
-  const int vbase_off = (4 * hh + ((s16 >> 1) & 3)) * V_PITCH + (s16 >> 3) * ROW_BYTES +
-                        16 * ((lane >> 4) & 1) + 8 * (s16 & 1);
+  unsigned vbase_off = lds_base + K_BYTES + (4 * hh + ((s16 >> 1) & 3)) * V_PITCH + (s16 >> 3) * ROW_BYTES +
+                       16 * ((lane >> 4) & 1) + 8 * (s16 & 1);
+  asm volatile("" : "+v"(kbase_off), "+v"(vbase_off));  // one register each through the loop
 
-  // ---- softmax state -------------------------------------------------------------------------
-  float sq = 1.f, sk = 1.f, sv = 1.f;
-  if (p.q_descale) sq = p.q_descale[b * p.ds_b + h * p.ds_h];
-  if (p.k_descale) sk = p.k_descale[b * p.ds_b + h * p.ds_h];
-  if (p.v_descale) sv = p.v_descale[b * p.ds_b + h * p.ds_h];
-  const float c = p.scale * sq * sk * kLog2e;
-  float m_used = -INFINITY;
-  float l_part = 0.f;
-  f32x16 oacc[4];
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
-
-  seek_tile(it0);
-  issue_tile(it0, 0);
-#pragma unroll
-  for (int ks = 0; ks < 2; ks++) asm volatile("" : "+v"(qf[ks]));
-
-  for (int t = it0; t < it1; t++) {
-    const int buf = (t - it0) & 1;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (t + 1 < it1) issue_tile(t + 1, buf ^ 1);
-
-    const XDIT_LDS u8* ktile = (const XDIT_LDS u8*)(smem + buf * BUF_BYTES) + kbase_off;
-    const XDIT_LDS u8* vtile = (const XDIT_LDS u8*)(smem + buf * BUF_BYTES + K_BYTES) + vbase_off;
-
-    // ---- S^T = K Q^T ---------------------------------------------------------------------
-    // Four MFMAs; MFMA m = 2 kb + ks takes the 32 bytes of its K row as two 16-byte reads.
-    f32x16 sacc[2];
-    {
-      constexpr int PD = kPrefetch;  // MFMAs whose two reads are in flight
-      constexpr int NM = 4;
-      const unsigned kaddr = (unsigned)(uintptr_t)ktile;
-      i32x4 klo[NM], khi[NM];
-      static_for<PD>([&](auto I) {
-        constexpr int m = I;
-        constexpr int off = (m / 2) * 4 * ROW_BYTES + (m % 2) * 64;
-        lds_read_b128<off>(klo[m], kaddr);
-        lds_read_b128<off + 16>(khi[m], kaddr);
-      });
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
-      static_for<NM>([&](auto I) {
-        constexpr int m = I;
-        constexpr int younger = 2 * ((m + PD <= NM ? PD : NM - m) - 1);
-        lds_wait2<younger>(klo[m], khi[m]);
-        i32x8 kf = __builtin_shufflevector(klo[m], khi[m], 0, 1, 2, 3, 4, 5, 6, 7);
-        sacc[m / 2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[m % 2], sacc[m / 2], 0, 0, 0, 0, 0, 0);
-        if constexpr (m + PD < NM) {
-          constexpr int n = m + PD;
-          constexpr int off = (n / 2) * 4 * ROW_BYTES + (n % 2) * 64;
-          lds_read_b128<off>(klo[n], kaddr);
-          lds_read_b128<off + 16>(khi[n], kaddr);
-        }
-      });
+  // ---- per segment: coordinates, Q fragments (2 contraction steps x 32 bytes), scales, first tile
+  int b, h, qt;
+  float c, sv;
+  i32x8 qf[2];
+  auto open_segment = [&](const Segment& sg) {
+    const int lane = lane_now(), l32 = lane & 31, hh = lane >> 5;
+    const int nq_tiles = pp->nq_tiles, H = pp->H;
+    const int bh = sg.tile / nq_tiles;
+    qt = sg.tile - bh * nq_tiles;
+    b = bh / H;
+    h = bh - b * H;
+    kv_k1 = (const u8*)pp->k + b * pp->ks_b + h * pp->ks_h;
+    kv_v1 = (const u8*)pp->v + b * pp->vs_b + h * pp->vs_h;
+    kss1 = (unsigned)pp->ks_s; vss1 = (unsigned)pp->vs_s;
+    keys1 = pp->Sk; keys2 = pp->Sk2;
+    if (keys2 > 0) {
+      kv_k2 = (const u8*)pp->k2 + b * pp->k2s_b + h * pp->k2s_h;
+      kv_v2 = (const u8*)pp->v2 + b * pp->v2s_b + h * pp->v2s_h;
+      kss2 = (unsigned)pp->k2s_s; vss2 = (unsigned)pp->v2s_s;
+    } else {
+      kv_k2 = kv_k1; kv_v2 = kv_v1; kss2 = kss1; vss2 = vss1;
     }
-
-    const int valid = (t < nt1) ? p.Sk - t * kKeysPerTile : p.Sk2 - (t - nt1) * kKeysPerTile;
-    if (valid < kKeysPerTile) {
+    float sq = 1.f, sk = 1.f;
+    sv = 1.f;
+    const int64_t ds = b * pp->ds_b + h * pp->ds_h;
+    if (pp->q_descale) sq = pp->q_descale[ds];
+    if (pp->k_descale) sk = pp->k_descale[ds];
+    if (pp->v_descale) sv = pp->v_descale[ds];
+    c = pp->scale * sq * sk * kLog2e;
+    const int Sq = pp->Sq;
+    const int qrow = qt * kRowsPerBlock + wave * kRowsPerWave + l32;
+    const int qrow_c = qrow < Sq ? qrow : Sq - 1;
+    const u8* qptr = (const u8*)pp->q + b * pp->qs_b + h * pp->qs_h + (int64_t)qrow_c * pp->qs_s + hh * 32;
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          int key = 32 * kb + 8 * (i >> 2) + 4 * hh + (i & 3);
-          if (key >= valid) sacc[kb][i] = -INFINITY;
-        }
+    for (int ks = 0; ks < 2; ks++) {
+      i32x4 lo = *(const i32x4*)(qptr + ks * 64);
+      i32x4 hi = *(const i32x4*)(qptr + ks * 64 + 16);
+      qf[ks] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
+    issue_tile(sg.it0, 0);
+  };
+  open_segment(seg);
 
-    // ---- online softmax ---------------------------------------------------------------
-    float mx = sacc[0][0];
-#pragma unroll
-    for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[0][i]);
-#pragma unroll
-    for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[1][i]);
-    mx = max_halves(mx);
-    const float m_new = fmaxf(m_used, mx);
-    const bool grow = (m_new - m_used) * c > kLazyRescaleLog2;
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-      const float alpha = fast_exp2((m_used - m_new) * c);
-      m_used = m_new;
-      l_part *= alpha;
-#pragma unroll
-      for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+  for (;;) {  // segments of this workgroup
+    const int cb = b, ch = h, cqt = qt;
+    const float cc = c, csv = sv;
+    TO* part_out = nullptr;
+    float* part_lse = nullptr;
+    if (seg.slot >= 0) {
+      part_out = (TO*)pp->ws_out + seg.slot * kRowsPerBlock * D;
+      part_lse = pp->ws_lse + seg.slot * kRowsPerBlock;
     }
-    const float mc = m_used * c - kPShift;
-    i32x8 pf;  // P^T: byte 16kb + i
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-      for (int i = 0; i < 16; i += 4) {
-        float p0 = fast_exp2(__builtin_fmaf(sacc[kb][i], c, -mc));
-        float p1 = fast_exp2(__builtin_fmaf(sacc[kb][i + 1], c, -mc));
-        float p2 = fast_exp2(__builtin_fmaf(sacc[kb][i + 2], c, -mc));
-        float p3 = fast_exp2(__builtin_fmaf(sacc[kb][i + 3], c, -mc));
-        l_part += (p0 + p1) + (p2 + p3);
-        int w;  // both halves are written below: no need to clear the register first
-        asm volatile("" : "=v"(w));
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, w, false);
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, w, true);
-        pf[4 * kb + (i >> 2)] = w;
-      }
-    }
-
-    // ---- O^T += V^T P^T ------------------------------------------------------------------
-    // Four MFMAs (d blocks); each takes its V^T operand as four transposing 8-byte reads.
-    {
-      constexpr int PD = kPrefetch;
-      constexpr int NM = 4;
-      const unsigned vaddr = (unsigned)(uintptr_t)vtile;
-      i32x2 vr[NM][4];
-      static_for<PD>([&](auto I) {
-        constexpr int m = I;
-        static_for<4>([&](auto R) {
-          constexpr int r = R;
-          lds_read_tr8_b64<r * 2 * ROW_BYTES + m * 32>(vr[m][r], vaddr);
-        });
-      });
-      static_for<NM>([&](auto I) {
-        constexpr int m = I;
-        constexpr int younger = 4 * ((m + PD <= NM ? PD : NM - m) - 1);
-        lds_wait4<younger>(vr[m][0], vr[m][1], vr[m][2], vr[m][3]);
-        i32x8 vf;
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          vf[2 * r] = vr[m][r][0];
-          vf[2 * r + 1] = vr[m][r][1];
-        }
-        oacc[m] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[m], 0, 0, 0, 0, 0, 0);
-        if constexpr (m + PD < NM) {
-          constexpr int n = m + PD;
-          static_for<4>([&](auto R) {
-            constexpr int r = R;
-            lds_read_tr8_b64<r * 2 * ROW_BYTES + n * 32>(vr[n][r], vaddr);
-          });
-        }
-      });
-    }
-  }
-
-  // ---- epilogue -----------------------------------------------------------------------------
-  const float l_tot = sum_halves(l_part);
-  const float inv = sv / l_tot;
-  const float lse = (m_used * c - kPShift + fast_log2(l_tot)) * kLn2;
-  if (qrow < p.Sq) {
-    TO* optr;
-    if (part_out != nullptr) optr = part_out + (wave * kRowsPerWave + l32) * D;
-    else optr = (TO*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s;
+    const int keys_1 = keys1, keys_2 = keys2;
+    float m_used = -INFINITY;
+    float l_part = 0.f;
+    f32x16 oacc[4];
 #pragma unroll
     for (int db = 0; db < 4; db++)
 #pragma unroll
-      for (int a = 0; a < 4; a++) {
-        typedef __attribute__((ext_vector_type(4))) TO vec4;
-        f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
-                   oacc[db][4 * a + 3] * inv};
-        vec4 ov = __builtin_convertvector(o, vec4);
-        *(vec4*)(optr + 32 * db + 8 * a + 4 * hh) = ov;
+      for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) asm volatile("" : "+v"(qf[ks]));
+
+    for (int t = seg.it0; t < seg.it1; t++) {
+      const int buf = (t - seg.it0) & 1;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (t + 1 < seg.it1) issue_tile(t + 1, buf ^ 1);
+
+      const unsigned kaddr = kbase_off + buf * BUF_BYTES;
+      const unsigned vaddr = vbase_off + buf * BUF_BYTES;
+
+      // ---- S^T = K Q^T ---------------------------------------------------------------------
+      // Four MFMAs; MFMA m = 2 kb + ks takes the 32 bytes of its K row as two 16-byte reads.
+      f32x16 sacc[2];
+      {
+        constexpr int PD = kPrefetch;  // MFMAs whose two reads are in flight
+        constexpr int NM = 4;
+        i32x4 klo[NM], khi[NM];
+        static_for<PD>([&](auto I) {
+          constexpr int m = I;
+          constexpr int off = (m / 2) * 4 * ROW_BYTES + (m % 2) * 64;
+          lds_read_b128<off>(klo[m], kaddr);
+          lds_read_b128<off + 16>(khi[m], kaddr);
+        });
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) sacc[kb][i] = 0.f;
+        static_for<NM>([&](auto I) {
+          constexpr int m = I;
+          constexpr int younger = 2 * ((m + PD <= NM ? PD : NM - m) - 1);
+          lds_wait2<younger>(klo[m], khi[m]);
+          i32x8 kf = __builtin_shufflevector(klo[m], khi[m], 0, 1, 2, 3, 4, 5, 6, 7);
+          sacc[m / 2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[m % 2], sacc[m / 2], 0, 0, 0, 0, 0, 0);
+          if constexpr (m + PD < NM) {
+            constexpr int n = m + PD;
+            constexpr int off = (n / 2) * 4 * ROW_BYTES + (n % 2) * 64;
+            lds_read_b128<off>(klo[n], kaddr);
+            lds_read_b128<off + 16>(khi[n], kaddr);
+          }
+        });
       }
-    if (hh == 0) {
-      if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
-      else if (p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = lse;
+
+      const int valid = (t < nt1) ? keys_1 - t * kKeysPerTile : keys_2 - (t - nt1) * kKeysPerTile;
+      if (valid < kKeysPerTile) {
+        const int hh = lane_now() >> 5;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            int key = 32 * kb + 8 * (i >> 2) + 4 * hh + (i & 3);
+            if (key >= valid) sacc[kb][i] = -INFINITY;
+          }
+      }
+
+      // ---- online softmax ---------------------------------------------------------------
+      float mx = sacc[0][0];
+#pragma unroll
+      for (int i = 1; i < 16; i++) mx = fmaxf(mx, sacc[0][i]);
+#pragma unroll
+      for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[1][i]);
+      mx = max_halves(mx);
+      const float m_new = fmaxf(m_used, mx);
+      const bool grow = (m_new - m_used) * cc > kLazyRescaleLog2;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        const float alpha = fast_exp2((m_used - m_new) * cc);
+        m_used = m_new;
+        l_part *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+      }
+      const float mc = m_used * cc - kPShift;
+      i32x8 pf;  // P^T: byte 16kb + i
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+        for (int i = 0; i < 16; i += 4) {
+          float p0 = fast_exp2(__builtin_fmaf(sacc[kb][i], cc, -mc));
+          float p1 = fast_exp2(__builtin_fmaf(sacc[kb][i + 1], cc, -mc));
+          float p2 = fast_exp2(__builtin_fmaf(sacc[kb][i + 2], cc, -mc));
+          float p3 = fast_exp2(__builtin_fmaf(sacc[kb][i + 3], cc, -mc));
+          l_part += (p0 + p1) + (p2 + p3);
+          int w;  // both halves are written below: no need to clear the register first
+          asm volatile("" : "=v"(w));
+          w = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, w, false);
+          w = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, w, true);
+          pf[4 * kb + (i >> 2)] = w;
+        }
+      }
+
+      // ---- O^T += V^T P^T ------------------------------------------------------------------
+      // Four MFMAs (d blocks); each takes its V^T operand as four transposing 8-byte reads.
+      {
+        constexpr int PD = kPrefetch;
+        constexpr int NM = 4;
+        i32x2 vr[NM][4];
+        static_for<PD>([&](auto I) {
+          constexpr int m = I;
+          static_for<4>([&](auto R) {
+            constexpr int r = R;
+            lds_read_tr8_b64<r * 2 * ROW_BYTES + m * 32>(vr[m][r], vaddr);
+          });
+        });
+        static_for<NM>([&](auto I) {
+          constexpr int m = I;
+          constexpr int younger = 4 * ((m + PD <= NM ? PD : NM - m) - 1);
+          lds_wait4<younger>(vr[m][0], vr[m][1], vr[m][2], vr[m][3]);
+          i32x8 vf;
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            vf[2 * r] = vr[m][r][0];
+            vf[2 * r + 1] = vr[m][r][1];
+          }
+          oacc[m] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[m], 0, 0, 0, 0, 0, 0);
+          if constexpr (m + PD < NM) {
+            constexpr int n = m + PD;
+            static_for<4>([&](auto R) {
+              constexpr int r = R;
+              lds_read_tr8_b64<r * 2 * ROW_BYTES + n * 32>(vr[n][r], vaddr);
+            });
+          }
+        });
+      }
     }
+    asm volatile("" : "+s"(pp));  // from here on the kernel arguments are read afresh
+
+    // ---- what comes next for this workgroup --------------------------------------------------
+    Segment next_seg;
+    bool more;
+    {
+      const WalkGeom g = walk_geom(pp);
+      unsigned* const range_counter = pp->split_counter;
+      if (walk.wants_claim(range_counter != nullptr)) {
+        __syncthreads();  // everyone has read the ticket of the previous claim
+        if (wave == 0 && lane_now() == 0) ticket = atomicAdd(range_counter, 1u);
+        __syncthreads();
+        walk.claimed(g, (unsigned)__builtin_amdgcn_readfirstlane((int)ticket));
+      }
+      more = walk.next(g, nt, next_seg);
+    }
+    __syncthreads();  // every wavefront is done with the K/V fragments of the last tile
+    if (more) open_segment(next_seg);  // Q fragments and first K/V tile (buffer 0) of the next segment
+
+    // ---- epilogue: rows through an LDS transpose, 64 columns at a time --------------------------
+    const int lane = lane_now(), l32 = lane & 31, hh = lane >> 5;
+    const int cqrow = cqt * kRowsPerBlock + wave * kRowsPerWave + l32;
+    const float l_tot = sum_halves(l_part);
+    const float inv = csv / l_tot;
+    const float lse = (m_used * cc - kPShift + fast_log2(l_tot)) * kLn2;
+    typedef __attribute__((ext_vector_type(4))) TO vec4;
+    typedef __attribute__((ext_vector_type(8))) TO vec8;
+    XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + BUF_BYTES + wave * kStageBytes;
+    const int row0 = cqt * kRowsPerBlock + wave * kRowsPerWave;
+    TO* obase;
+    int64_t ostride;
+    int rows_live = kRowsPerWave;
+    if (part_out != nullptr) {
+      obase = part_out + (int64_t)(wave * kRowsPerWave) * D;
+      ostride = D;
+    } else {
+      obase = (TO*)pp->out + cb * pp->os_b + ch * pp->os_h + (int64_t)row0 * pp->os_s;
+      ostride = pp->os_s;
+      rows_live = pp->Sq - row0;  // may be <= 0 or above 32
+    }
+    const int rd_row = lane >> 3;          // + 8r
+    const int rd_col = (lane & 7) * 8;     // element column within the 64-column pass
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+#pragma unroll
+      for (int dbl = 0; dbl < 2; dbl++) {
+        const int db = 2 * half + dbl;
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+          f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                     oacc[db][4 * a + 3] * inv};
+          *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int row = rd_row + 8 * r;
+        const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
+        if (row < rows_live) __builtin_nontemporal_store(x, (vec8*)(obase + row * ostride + 64 * half + rd_col));
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    if (hh == 0 && cqrow < pp->Sq) {
+      if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
+      else if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = lse;
+    }
+    if (!more) break;
+    seg = next_seg;
   }
 }
 
 template <typename TO, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 8 ? 2 : 3) void attn_fwd_fp8_kernel(const AttnParams p) {
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF_BYTES];
-  run_workgroup<TO, kRowsPerWave * NW, D>(p, [&](int tile, int it0, int it1, TO* part_out, float* part_lse) {
-    attn_segment_fp8<TO, NW>(p, smem, tile, it0, it1, part_out, part_lse);
-  });
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // [K tile | V tile] [K tile | V tile, or output staging]
+  attn_workgroup_fp8<TO, NW>(smem);
 }
 
 // Workgroups of NW wavefronts resident at once (3 wavefronts per SIMD by registers; 2 for NW = 8).
@@ -330,8 +408,16 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
   bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1), rows, D, 2);
   launch_counter_reset(q, stream);
+  static std::atomic<bool> lds_ready[kMaxDevices];
+  constexpr int lds = lds_bytes<NW>();
+  const int slot = current_device_slot();
+  if (lds > 65536 && !lds_ready[slot].load(std::memory_order_relaxed)) {  // > 64 KiB of dynamic LDS must be enabled once per kernel and device
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_fp8_kernel<TO, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return e;
+    lds_ready[slot].store(true, std::memory_order_relaxed);
+  }
   dim3 grid(split_grid(q));
-  hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW>), grid, dim3(64 * NW), 0, stream, q);
+  hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW>), grid, dim3(64 * NW), lds, stream, q);
   if (q.split_units) {
     const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
     const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));

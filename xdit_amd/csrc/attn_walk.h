@@ -150,9 +150,8 @@ XDIT_HD int shared_tile_parts(const P& p, int nt, int r) {
 }
 
 // Thread -> (row, first 8-element chunk) map of the merge kernel.  A row of `cpr` chunks is held
-// by lanes_per_row = min(cpr, 64) adjacent lanes of ONE wavefront (lane j of the row takes chunks
-// j, j + lanes_per_row, ...), a wavefront holds rows_per_wave = 64 / lanes_per_row whole rows and
-// its remaining lanes idle.  A row never spans two wavefronts: every lane of a row reads the
+// by cpr adjacent lanes of ONE wavefront (cpr <= 64, i.e. head_dim <= 512), a wavefront holds
+// rows_per_wave = 64 / cpr whole rows and its remaining lanes idle.  A row never spans two wavefronts: every lane of a row reads the
 // row's log-sum-exp before the row's first lane overwrites it, which only program order inside
 // one wavefront guarantees.
 struct MergeMap {

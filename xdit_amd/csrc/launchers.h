@@ -38,6 +38,15 @@ struct QuantParams {
   int per_tensor;
   int had_block;    // Hadamard rotation block along head_dim (<= 1: none)
   float had_scale;  // 1/sqrt(had_block) in fp32; the kernel rounds it to the input dtype
+  // optional second tensor (B,H,S2,D) quantised with the scales of the first
+  const void* x2;
+  void* y2;
+  int64_t x2s_b, x2s_h, x2s_s;
+  int64_t y2s_b, y2s_h, y2s_s;
+  int S2;
+  // optional scratch: partial_slots floats, one per workgroup of the abs-max pass
+  float* partials;
+  int64_t partial_slots;
 };
 
 // Parameters of one prologue launch (RMSNorm + rotary embedding + re-layout of Q or K).

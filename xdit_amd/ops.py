@@ -341,11 +341,16 @@ def lse_merge(acc_out, acc_lse, block_out, block_lse, first=False, final_out=Non
     return acc_out, acc_lse
 
 
-def fp8_quant(x, per_tensor=False, scale=None, hadamard_block=0):
+_QUANT_SCRATCH = {}
+
+
+def fp8_quant(x, per_tensor=False, scale=None, hadamard_block=0, x2=None):
     """Abs-max fp8 quantiser on a logical BHSD tensor -> (y float8_e4m3fn BHSD-contiguous,
     descale (B,H) fp32).  `per_tensor` takes one abs-max over the whole tensor (the reference's
     per_tensor_quant); `scale` (a one-element fp32 tensor) is a static scale; `hadamard_block`
-    (a power of two dividing head_dim) rotates the rows by a block Hadamard matrix first."""
+    (a power of two dividing head_dim) rotates the rows by a block Hadamard matrix first.
+    `x2` (logical (B,H,S2,D), e.g. the joint keys) is quantised with the same scales, the abs-max
+    taken over both tensors; the result is then (y, y2, descale)."""
     device = x.device
     _check4("x", x, device)
     B, H, S, D = x.shape
@@ -358,14 +363,31 @@ def fp8_quant(x, per_tensor=False, scale=None, hadamard_block=0):
     a.hadamard_block = int(hadamard_block)
     a.B, a.H, a.D, a.S = B, H, D, S
     a.x, a.y, a.descale = x.data_ptr(), y.data_ptr(), descale.data_ptr()
+    y2 = None
+    if x2 is not None:
+        _check4("x2", x2, device)
+        if x2.shape[0] != B or x2.shape[1] != H or x2.shape[3] != D or x2.dtype != x.dtype:
+            raise ValueError("x2 %s does not match x %s" % (tuple(x2.shape), tuple(x.shape)))
+        y2 = torch.empty(tuple(x2.shape), dtype=torch.float8_e4m3fn, device=device)
+        if x2.shape[2] > 0:
+            a.S2 = x2.shape[2]
+            a.x2, a.y2 = x2.data_ptr(), y2.data_ptr()
+            a.x2_stride, a.y2_stride = _strides(x2), _strides(y2)
     if scale is not None:
         scale = scale.to(device=device, dtype=torch.float32).reshape(1).contiguous()
         a.scale_in = scale.data_ptr()
     a.x_stride, a.y_stride = _strides(x), _strides(y)
-    a.stream = _stream(device)
+    stream = _stream(device)
+    a.stream = stream
+    need = 4 * max(4096, B * H)
+    buf = _QUANT_SCRATCH.get((device, stream))
+    if buf is None or buf.numel() < need:
+        buf = torch.empty(need, dtype=torch.uint8, device=device)
+        _QUANT_SCRATCH[(device, stream)] = buf
+    a.scratch, a.scratch_bytes = buf.data_ptr(), buf.numel()
     with _on_device(device):
         _lib.check(_lib.lib().xdit_fp8_quant(ctypes.byref(a)))
-    return y, descale
+    return (y, descale) if x2 is None else (y, y2, descale)
 
 
 _NORM_MODES = {None: _lib.NORM_NONE, "none": _lib.NORM_NONE, "head": _lib.NORM_HEAD, "token": _lib.NORM_TOKEN}
