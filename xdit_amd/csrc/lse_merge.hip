@@ -77,23 +77,22 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const MergeParams p, con
   float* ao_row = p.acc_out + b * p.ao_b + h * p.ao_h + s * p.ao_s;
   const TB* bo_row = (const TB*)p.block_out + b * p.bo_b + h * p.bo_h + s * p.bo_s;
 
-  // the row's chunk is requested before the two log-sum-exps, so that one round trip to memory
-  // covers them all (head_dim <= 512: a lane holds one chunk)
-  const int col = chunk0 * 8;
+  const int col = chunk0 * 8;  // head_dim <= 512: a lane holds one chunk
   float xb[8], xo[8];
   Load8<TB>::ld(bo_row + col, xb);
-  if (!p.first) Load8<float>::ld(ao_row + col, xo);
   const float blse = *bl;
-  float new_lse = blse;
+  float new_lse;
   if (p.first) {
 #pragma unroll
     for (int i = 0; i < 8; i++) xo[i] = xb[i];
+    new_lse = blse;
   } else {
+    Load8<float>::ld(ao_row + col, xo);
     const float lse = *al;  // read by every lane of the row before its first lane stores below
     const float w = sigmoid(blse - lse);
-    new_lse = lse - log_sigmoid(lse - blse);
 #pragma unroll
     for (int i = 0; i < 8; i++) xo[i] = fold_value(xo[i], xb[i], w);
+    new_lse = lse - log_sigmoid(lse - blse);
   }
   Load8<float>::st(ao_row + col, xo);
   if (HAS_FINAL) {
