@@ -212,7 +212,7 @@ int xdit_lse_merge(const xdit_merge_args* args);
 /*
  * One ring step in one launch: the forward of xdit_attn_fwd on this step's keys/values, folded
  * into the fp32 accumulator (acc_out, acc_lse) in the kernel's epilogue with the arithmetic of
- * xdit_lse_merge.  The block's rows are rounded to `dtype` before the fold, as if they had gone
+ * xdit_lse_merge.  The block's rows are rounded to `out_dtype` before the fold, as if they had gone
  * through a block_out tensor, so the result equals xdit_attn_fwd + xdit_lse_merge bit for bit
  * while the block is never written to memory and the accumulator is touched once.
  *   first != 0            initialise the accumulator from this block (acc_out is not read)
@@ -221,8 +221,9 @@ int xdit_lse_merge(const xdit_merge_args* args);
  *   discard_acc_out != 0  acc_out is read but not written back (last step: `out` and acc_lse
  *                         carry the result); needs args->out
  * acc_out is logical (B,H,Sq,D) fp32, acc_lse logical (B,H,Sq) fp32 with its own strides (the
- * (B,S,H,1) accumulator of the legacy ring maps without a copy).  bf16 / fp16 inputs with
- * head_dim a multiple of 8 up to 128; XDIT_ERR_UNSUPPORTED otherwise (use the two calls).
+ * (B,S,H,1) accumulator of the legacy ring maps without a copy).  bf16 / fp16 / fp32 inputs with
+ * head_dim a multiple of 8 up to 128, fp8 inputs with head_dim 128; XDIT_ERR_UNSUPPORTED
+ * otherwise (use the two calls).
  * args->workspace is not used.
  * Replaces, per ring step: the kernel call at ring_flash_attn.py:123-134, update_out_and_lse at
  * :138 and, on the last step, the cast at :145.

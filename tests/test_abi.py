@@ -227,7 +227,7 @@ def test_fused_ring_step_rejects_bad_arguments():
     r.acc_out, r.acc_lse = 0x2000, 0x3000
     r.acc_out_stride = _lib.Strides(a.H * a.Sq * a.D, a.Sq * a.D, a.D)
     r.acc_lse_stride = _lib.Strides(a.H * a.Sq, a.Sq, 1)
-    f8 = _attn_args(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16)
+    f8 = _attn_args(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16, D=64)  # the fp8 ring step needs head_dim 128
     assert L.xdit_attn_fwd_accumulate(ctypes.byref(f8), ctypes.byref(r)) == _lib.XDIT_ERR_UNSUPPORTED and "fused ring step" in _lib.last_error()
     r.acc_out = 0x2004
     assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "acc_out" in _lib.last_error()

@@ -86,6 +86,29 @@ def test_attn_generic_path_vs_oracle(gpu, dtype, D, Sq, Sk):
     assert _err(o, ro) <= TOL[dtype][0] and _err(l, rl) <= TOL[dtype][1]
 
 
+@pytest.mark.parametrize("cus", [1, 0])
+@pytest.mark.parametrize("D", [72, 8, 128, 40])
+@pytest.mark.parametrize("Sq,Sk,Sk2", [(1, 1, 0), (70, 33, 0), (130, 200, 45), (64, 32, 1), (257, 64, 65), (200, 31, 100)])
+def test_attn_fp32_both_workgroup_forms_vs_oracle(gpu, monkeypatch, cus, D, Sq, Sk, Sk2):
+    """The fp32 kernel in both forms: planned for one compute unit these problems keep 128-row
+    workgroups with 32-key tiles; planned for the device's own count they are small enough to take
+    64-row workgroups whose wavefront pairs split 64-key tiles and fold through LDS (key halves
+    that are empty or ragged included), with and without a second KV segment."""
+    monkeypatch.setitem(ops.TUNING, "cu_count", cus)
+    g = torch.Generator().manual_seed(D * 1000 + Sq + Sk2)
+    q = torch.randn(1, 3, Sq, D, generator=g)
+    k, v = torch.randn(1, 3, Sk, D, generator=g), torch.randn(1, 3, Sk, D, generator=g)
+    kw = {}
+    kall, vall = k, v
+    if Sk2:
+        k2, v2 = torch.randn(1, 3, Sk2, D, generator=g), torch.randn(1, 3, Sk2, D, generator=g)
+        kall, vall = torch.cat([k, k2], 2), torch.cat([v, v2], 2)
+        kw = dict(k2=_layout(k2, "bshd", gpu), v2=v2.to(gpu))
+    ro, rl = O.attn_fwd_ref(q, kall, vall)
+    o, l = ops.attn_fwd(q.to(gpu), _layout(k, "bshd", gpu), v.to(gpu), **kw)
+    assert _err(o, ro) <= 2e-5 and _err(l, rl) <= 2e-5
+
+
 def test_tiny_bruteforce_golden(gpu):
     z = np.load(os.path.join(GOLD, "tiny_bruteforce.npz"))
     for n in (2, 3, 4):  # the head_dim 8 cases
@@ -630,6 +653,81 @@ def test_fused_ring_step_equals_forward_plus_merge(gpu, force_rows, dtype, D, la
             oo, ol = (ro.to(dtype).double(), rl) if oo is None else O.merge_ref(oo, ol, ro.to(dtype), rl)
         assert torch.equal(fin, ref_fin)
         assert _err(acc_o, oo) <= 2e-2 and _err(acc_l, ol) <= 1e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cus", [1, 0])
+@pytest.mark.parametrize("D", [72, 128, 16])
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+def test_fused_ring_step_fp32_equals_forward_plus_merge(gpu, monkeypatch, cus, D, layout):
+    """The fp32 ring step (both workgroup forms of the fp32 kernel) against forward + merge, bit
+    for bit, and against the oracle's fold."""
+    monkeypatch.setitem(ops.TUNING, "cu_count", cus)
+    B, H, Sq = 2, 2, 150
+    g = torch.Generator().manual_seed(D + 7)
+    q = torch.randn(B, H, Sq, D, generator=g)
+    chunks = [(torch.randn(B, H, n, D, generator=g), torch.randn(B, H, n, D, generator=g)) for n in (97, 32, 130)]
+    qd = _layout(q, layout, gpu)
+    acc_o = _layout(torch.full((B, H, Sq, D), float("nan")), layout, gpu)
+    acc_l = torch.full((B, Sq, H, 1), float("nan"), device=gpu).squeeze(-1).transpose(1, 2)
+    ref_o, ref_l = torch.empty(B, H, Sq, D, device=gpu), torch.empty(B, H, Sq, device=gpu)
+    fin = torch.empty(B, H, Sq, D, device=gpu)
+    oo = ol = None
+    for i, (k, v) in enumerate(chunks):
+        kd, vd = _layout(k, layout, gpu), _layout(v, layout, gpu)
+        last = i + 1 == len(chunks)
+        ops.attn_fwd_accumulate(qd, kd, vd, acc_o, acc_l, first=i == 0, final_out=fin if last else None)
+        bo, bl = ops.attn_fwd(qd, kd, vd)
+        ops.lse_merge(ref_o, ref_l, bo, bl, first=i == 0)
+        assert torch.equal(acc_o, ref_o) and torch.equal(acc_l, ref_l), i
+        ro, rl = O.attn_fwd_ref(q, k, v)
+        oo, ol = (ro, rl) if oo is None else O.merge_ref(oo, ol, ro, rl)
+    assert torch.equal(fin, ref_o)
+    assert _err(acc_o, oo) <= 2e-5 and _err(acc_l, ol) <= 2e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+def test_fused_ring_step_fp8_equals_forward_plus_merge(gpu, force_rows, out_dtype, layout):
+    """The fp8 ring step in every workgroup shape against forward + merge, bit for bit, with a
+    second KV segment on one step; and against the oracle's fold of the dequantised inputs."""
+    B, H, Sq, D = 1, 3, 333, 128
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, H, Sq, D, generator=g)
+    chunks = [(torch.randn(B, H, n, D, generator=g), torch.randn(B, H, n, D, generator=g)) for n in (257, 64, 130)]
+    jk, jv = torch.randn(B, H, 50, D, generator=g), torch.randn(B, H, 50, D, generator=g)
+    q8, qs = ops.fp8_quant(q.to(gpu))
+    q8l = _layout(q8.cpu().view(torch.uint8), layout, gpu).view(torch.float8_e4m3fn)
+    quant = []
+    for k, v in chunks:
+        k8, j8, ks = ops.fp8_quant(k.to(gpu), x2=jk.to(gpu))
+        v8, w8, vs = ops.fp8_quant(v.to(gpu), x2=jv.to(gpu))
+        quant.append((k8, v8, j8, w8, ks, vs))
+    for rows in (128, 256, 384):
+        force_rows(rows)
+        acc_o = _layout(torch.full((B, H, Sq, D), float("nan")), layout, gpu)
+        acc_l = torch.full((B, Sq, H, 1), float("nan"), device=gpu).squeeze(-1).transpose(1, 2)
+        ref_o, ref_l = torch.empty(B, H, Sq, D, device=gpu), torch.empty(B, H, Sq, device=gpu)
+        fin = torch.empty(B, H, Sq, D, dtype=out_dtype, device=gpu)
+        ref_fin = torch.empty_like(fin)
+        oo = ol = None
+        for i, (k8, v8, j8, w8, ks, vs) in enumerate(quant):
+            last = i + 1 == len(quant)
+            kw = dict(q_descale=qs, k_descale=ks, v_descale=vs, out_dtype=out_dtype)
+            if i == 1:
+                kw.update(k2=j8, v2=w8)
+            ops.attn_fwd_accumulate(q8l, k8, v8, acc_o, acc_l, first=i == 0, final_out=fin if last else None, **kw)
+            bo, bl = ops.attn_fwd(q8l, k8, v8, **kw)
+            ops.lse_merge(ref_o, ref_l, bo, bl, first=i == 0, final_out=ref_fin if last else None)
+            assert torch.equal(acc_o, ref_o) and torch.equal(acc_l, ref_l), (rows, i)
+            kd, vd = O.dequant(k8.cpu(), ks.cpu()), O.dequant(v8.cpu(), vs.cpu())
+            if i == 1:
+                kd, vd = torch.cat([kd, O.dequant(j8.cpu(), ks.cpu())], 2), torch.cat([vd, O.dequant(w8.cpu(), vs.cpu())], 2)
+            ro, rl = O.attn_fwd_ref(O.dequant(q8.cpu(), qs.cpu()), kd, vd)
+            oo, ol = (ro.to(out_dtype).double(), rl) if oo is None else O.merge_ref(oo, ol, ro.to(out_dtype), rl)
+        assert torch.equal(fin, ref_fin)
+        assert _err(acc_o, oo) <= 6e-2 and _err(acc_l, ol) <= 1e-3
 
 
 @pytest.mark.gpu

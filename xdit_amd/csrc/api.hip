@@ -225,8 +225,8 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   if (acc != nullptr) {
     if (acc->struct_size != sizeof(xdit_ring_acc))
       return fail(XDIT_ERR_INVALID_ARG, "acc struct_size %u != %zu (ABI mismatch)", acc->struct_size, sizeof(xdit_ring_acc));
-    if (!mfma16_path(a))
-      return fail(XDIT_ERR_UNSUPPORTED, "the fused ring step needs bf16 or fp16 inputs with head_dim at most 128");
+    if (a->dtype == XDIT_DTYPE_FP8_E4M3FN ? a->D != 128 : a->D > 128)
+      return fail(XDIT_ERR_UNSUPPORTED, "the fused ring step needs head_dim at most 128 (fp8: 128), got %d", a->D);
     if ((rc = check_tensor("acc_out", acc->acc_out, acc->acc_out_stride, 4, a->D))) return rc;
     if (acc->acc_lse == nullptr) return fail(XDIT_ERR_INVALID_ARG, "acc_lse is NULL");
     if (acc->acc_lse_stride.b < 0 || acc->acc_lse_stride.h < 0 || acc->acc_lse_stride.s <= 0)

@@ -44,7 +44,7 @@ constexpr int kPrefetch = 2;
 // Output staging block of a wavefront in the epilogue: 32 rows of 64 16-bit columns, rows 8 bytes
 // apart from a multiple of 128 so that the 8-byte writes of the 32 lanes of a half hit 32 banks.
 constexpr int kStagePitch = 64 * 2 + 8;
-constexpr int kStageBytes = kRowsPerWave * kStagePitch;
+constexpr int kStageBytes = kRowsPerWave * kStagePitch + kRowsPerWave * 4;  // + one fp32 per row (ring step)
 // LDS of a workgroup: the first K/V buffer, then a region that holds the second K/V buffer during
 // the KV loop and the output staging blocks of the wavefronts in the epilogue.
 template <int NW>
@@ -57,7 +57,10 @@ constexpr int lds_bytes() { return BUF_BYTES + (BUF_BYTES > NW * kStageBytes ? B
 // registers), the Q fragments and the first K/V tile of a workgroup's next segment are requested
 // ahead of the epilogue of the current one, and the rows leave through an LDS transpose as
 // whole 128-byte lines.
-template <typename TO, int NW>
+// FUSED: the ring step; the block (rounded to TO, what a block_out tensor would have held) is
+// folded into the fp32 accumulator with the arithmetic of the merge kernel, so that the result
+// equals forward + merge bit for bit; such a launch has whole query tiles only.
+template <typename TO, int NW, bool FUSED>
 __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
   typedef unsigned char u8;
   ParamsPtr pp = (ParamsPtr)__builtin_amdgcn_kernarg_segment_ptr();
@@ -345,83 +348,152 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
     typedef __attribute__((ext_vector_type(8))) TO vec8;
     XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + BUF_BYTES + wave * kStageBytes;
     const int row0 = cqt * kRowsPerBlock + wave * kRowsPerWave;
-    TO* obase;
-    int64_t ostride;
-    int rows_live = kRowsPerWave;
-    if (part_out != nullptr) {
-      obase = part_out + (int64_t)(wave * kRowsPerWave) * D;
-      ostride = D;
-    } else {
-      obase = (TO*)pp->out + cb * pp->os_b + ch * pp->os_h + (int64_t)row0 * pp->os_s;
-      ostride = pp->os_s;
-      rows_live = pp->Sq - row0;  // may be <= 0 or above 32
-    }
-    const int rd_row = lane >> 3;          // + 8r
-    const int rd_col = (lane & 7) * 8;     // element column within the 64-column pass
+    if constexpr (!FUSED) {
+      TO* obase;
+      int64_t ostride;
+      int rows_live = kRowsPerWave;
+      if (part_out != nullptr) {
+        obase = part_out + (int64_t)(wave * kRowsPerWave) * D;
+        ostride = D;
+      } else {
+        obase = (TO*)pp->out + cb * pp->os_b + ch * pp->os_h + (int64_t)row0 * pp->os_s;
+        ostride = pp->os_s;
+        rows_live = pp->Sq - row0;  // may be <= 0 or above 32
+      }
+      const int rd_row = lane >> 3;          // + 8r
+      const int rd_col = (lane & 7) * 8;     // element column within the 64-column pass
 #pragma unroll
-    for (int half = 0; half < 2; half++) {
+      for (int half = 0; half < 2; half++) {
 #pragma unroll
-      for (int dbl = 0; dbl < 2; dbl++) {
-        const int db = 2 * half + dbl;
+        for (int dbl = 0; dbl < 2; dbl++) {
+          const int db = 2 * half + dbl;
 #pragma unroll
-        for (int a = 0; a < 4; a++) {
-          f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
-                     oacc[db][4 * a + 3] * inv};
-          *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+          for (int a = 0; a < 4; a++) {
+            f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                       oacc[db][4 * a + 3] * inv};
+            *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+          }
         }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int row = rd_row + 8 * r;
-        const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
-        if (row < rows_live) __builtin_nontemporal_store(x, (vec8*)(obase + row * ostride + 64 * half + rd_col));
+        for (int r = 0; r < 4; r++) {
+          const int row = rd_row + 8 * r;
+          const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
+          if (row < rows_live) __builtin_nontemporal_store(x, (vec8*)(obase + row * ostride + 64 * half + rd_col));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-    }
-    if (hh == 0 && cqrow < pp->Sq) {
-      if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
-      else if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = lse;
+      if (hh == 0 && cqrow < pp->Sq) {
+        if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
+        else if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = lse;
+      }
+    } else {
+      // the block goes through the same LDS transpose, so that the accumulator is read and written
+      // in whole rows; the weight of each row's fold travels with it
+      XDIT_LDS float* wrow = (XDIT_LDS float*)(stage + kRowsPerWave * kStagePitch);
+      const bool first = pp->acc_first != 0;
+      float* alp = pp->acc_lse + cb * pp->al_b + ch * pp->al_h + (int64_t)cqrow * pp->al_s;
+      float w = 0.f, new_lse = lse;
+      if (!first && cqrow < pp->Sq) {
+        const float la = *alp;
+        w = sigmoid(lse - la);
+        new_lse = la - log_sigmoid(la - lse);
+      }
+      if (hh == 0) wrow[l32] = w;
+      float* abase = pp->acc_out + cb * pp->ao_b + ch * pp->ao_h + (int64_t)row0 * pp->ao_s;
+      TO* obase = pp->out != nullptr ? (TO*)pp->out + cb * pp->os_b + ch * pp->os_h + (int64_t)row0 * pp->os_s : nullptr;
+      const int rows_live = pp->Sq - row0;
+      const int rd_row = lane >> 3;
+      const int rd_col = (lane & 7) * 8;
+#pragma unroll
+      for (int half = 0; half < 2; half++) {
+#pragma unroll
+        for (int dbl = 0; dbl < 2; dbl++) {
+          const int db = 2 * half + dbl;
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            f32x4 o = {oacc[db][4 * a] * inv, oacc[db][4 * a + 1] * inv, oacc[db][4 * a + 2] * inv,
+                       oacc[db][4 * a + 3] * inv};
+            *(XDIT_LDS vec4*)(stage + l32 * kStagePitch + (32 * dbl + 8 * a + 4 * hh) * 2) = __builtin_convertvector(o, vec4);
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int row = rd_row + 8 * r;
+          const int col = 64 * half + rd_col;
+          const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
+          const float wr = wrow[row];
+          if (row < rows_live) {
+            float* aptr = abase + row * pp->ao_s + col;
+            f32x4 m0, m1;
+#pragma unroll
+            for (int e = 0; e < 4; e++) { m0[e] = (float)x[e]; m1[e] = (float)x[4 + e]; }
+            if (!first) {
+              const f32x4 a0 = *(const f32x4*)aptr, a1 = *(const f32x4*)(aptr + 4);
+#pragma unroll
+              for (int e = 0; e < 4; e++) { m0[e] = fold_value(a0[e], m0[e], wr); m1[e] = fold_value(a1[e], m1[e], wr); }
+            }
+            if (pp->acc_store) { *(f32x4*)aptr = m0; *(f32x4*)(aptr + 4) = m1; }
+            if (obase != nullptr) {
+              vec8 y;
+#pragma unroll
+              for (int e = 0; e < 4; e++) { y[e] = (TO)m0[e]; y[4 + e] = (TO)m1[e]; }
+              *(vec8*)(obase + row * pp->os_s + col) = y;
+            }
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+      if (hh == 0 && cqrow < pp->Sq) {
+        *alp = new_lse;
+        if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = new_lse;
+      }
     }
     if (!more) break;
     seg = next_seg;
   }
 }
 
-template <typename TO, int NW>
+template <typename TO, int NW, bool FUSED>
 __global__ __launch_bounds__(64 * NW, NW == 8 ? 2 : 3) void attn_fwd_fp8_kernel(const AttnParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // [K tile | V tile] [K tile | V tile, or output staging]
-  attn_workgroup_fp8<TO, NW>(smem);
+  attn_workgroup_fp8<TO, NW, FUSED>(smem);
 }
 
 // Workgroups of NW wavefronts resident at once (3 wavefronts per SIMD by registers; 2 for NW = 8).
 static int resident_workgroups(int NW, int planned_cus) { return resident_cus(planned_cus) * (NW == 4 ? 3 : 1); }
 
-template <typename TO, int NW>
+template <typename TO, int NW, bool FUSED>
 static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   AttnParams q = p;
   constexpr int rows = kRowsPerWave * NW;
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1), rows, D, 2);
-  launch_counter_reset(q, stream);
+  // the ring step folds in the epilogue of whole query tiles: no shared last round
+  bind_workspace(q, p, FUSED ? 0 : plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1), rows, D, 2);
+  if constexpr (!FUSED) launch_counter_reset(q, stream);
   static std::atomic<bool> lds_ready[kMaxDevices];
   constexpr int lds = lds_bytes<NW>();
   const int slot = current_device_slot();
   if (lds > 65536 && !lds_ready[slot].load(std::memory_order_relaxed)) {  // > 64 KiB of dynamic LDS must be enabled once per kernel and device
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_fp8_kernel<TO, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_fp8_kernel<TO, NW, FUSED>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     lds_ready[slot].store(true, std::memory_order_relaxed);
   }
   dim3 grid(split_grid(q));
-  hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW>), grid, dim3(64 * NW), lds, stream, q);
-  if (q.split_units) {
-    const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-    const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
-    hipLaunchKernelGGL((attn_combine_kernel<TO, D>), cgrid, dim3(256), 0, stream, q, rows, nt, split_counters(q));
+  hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW, FUSED>), grid, dim3(64 * NW), lds, stream, q);
+  if constexpr (!FUSED) {
+    if (q.split_units) {
+      const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
+      const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
+      hipLaunchKernelGGL((attn_combine_kernel<TO, D>), cgrid, dim3(256), 0, stream, q, rows, nt, split_counters(q));
+    }
   }
   return hipGetLastError();
 }
@@ -441,11 +513,17 @@ static size_t workspace_one(const AttnParams& p, AttnParams* plan) {
 }  // namespace fp8path
 
 // rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12 wavefronts sharing each K/V tile).
-hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream) {
+template <bool FUSED>
+static hipError_t launch_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream) {
   using namespace fp8path;
-  if (rows_per_block == 384) return out_is_fp16 ? launch_one<_Float16, 12>(p, stream) : launch_one<__bf16, 12>(p, stream);
-  if (rows_per_block == 256) return out_is_fp16 ? launch_one<_Float16, 8>(p, stream) : launch_one<__bf16, 8>(p, stream);
-  return out_is_fp16 ? launch_one<_Float16, 4>(p, stream) : launch_one<__bf16, 4>(p, stream);
+  if (rows_per_block == 384) return out_is_fp16 ? launch_one<_Float16, 12, FUSED>(p, stream) : launch_one<__bf16, 12, FUSED>(p, stream);
+  if (rows_per_block == 256) return out_is_fp16 ? launch_one<_Float16, 8, FUSED>(p, stream) : launch_one<__bf16, 8, FUSED>(p, stream);
+  return out_is_fp16 ? launch_one<_Float16, 4, FUSED>(p, stream) : launch_one<__bf16, 4, FUSED>(p, stream);
+}
+
+// p.acc_out set: the ring step (fold into the fp32 accumulator in the epilogue).
+hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream) {
+  return p.acc_out != nullptr ? launch_fp8<true>(p, out_is_fp16, rows_per_block, stream) : launch_fp8<false>(p, out_is_fp16, rows_per_block, stream);
 }
 
 size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan) {

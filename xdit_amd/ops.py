@@ -287,20 +287,29 @@ def launch_plan(q, k, k2=None, deterministic=None):
 
 
 def fused_ring_step_supported(q):
-    """Whether `attn_fwd_accumulate` takes these queries (bf16 / fp16, head_dim a multiple of 8 up to 128)."""
-    return q.dtype in (torch.bfloat16, torch.float16) and q.shape[-1] % 8 == 0 and 0 < q.shape[-1] <= 128
+    """Whether `attn_fwd_accumulate` takes these queries (bf16 / fp16 / fp32 with head_dim a multiple
+    of 8 up to 128, fp8 with head_dim 128)."""
+    if q.dtype == torch.float8_e4m3fn:
+        return q.shape[-1] == 128
+    return q.dtype in (torch.bfloat16, torch.float16, torch.float32) and q.shape[-1] % 8 == 0 and 0 < q.shape[-1] <= 128
 
 
 def attn_fwd_accumulate(q, k, v, acc_out, acc_lse, first=False, final_out=None, discard_acc_out=False,
-                        softmax_scale=None, k2=None, v2=None):
+                        softmax_scale=None, k2=None, v2=None, q_descale=None, k_descale=None, v_descale=None,
+                        out_dtype=None):
     """One ring step in one launch: attention of q over (k, v) [+ (k2, v2)] folded into the fp32
     accumulator (acc_out logical BHSD, acc_lse logical BHS; any strides) exactly as `attn_fwd`
     followed by `lse_merge` would, without the block ever reaching memory.  `first` initialises
-    the accumulator; `final_out` (logical BHSD, q's dtype) also receives the merged rows;
-    `discard_acc_out` skips the write-back of acc_out (last step).  Returns (acc_out, acc_lse)."""
+    the accumulator; `final_out` (logical BHSD, q's dtype; bf16 or fp16 for fp8 inputs) also
+    receives the merged rows; `discard_acc_out` skips the write-back of acc_out (last step).
+    fp8 inputs take (B, H) fp32 descales and `out_dtype` (bf16 by default), the dtype the block is
+    rounded to before the fold.  Returns (acc_out, acc_lse)."""
     if discard_acc_out and final_out is None:
         raise ValueError("discard_acc_out needs final_out")
+    if out_dtype is None and final_out is not None:
+        out_dtype = final_out.dtype
     attn_fwd(q, k, v, softmax_scale=softmax_scale, k2=k2, v2=v2, out=final_out, return_lse=False,
+             q_descale=q_descale, k_descale=k_descale, v_descale=v_descale, out_dtype=out_dtype,
              _acc=(acc_out, acc_lse, bool(first), bool(discard_acc_out)))
     return acc_out, acc_lse
 

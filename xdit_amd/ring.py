@@ -124,7 +124,7 @@ def xdit_ring_flash_attn_forward(process_group, q, k, v, softmax_scale, dropout_
     out = None
     lse = None
     final = None
-    # bf16 / fp16 at head_dim up to 128: every step is one launch that folds its block into the
+    # head_dim up to 128 (fp8: 128): every step is one launch that folds its block into the
     # accumulator in the kernel's epilogue (same bits as kernel call + update_out_and_lse).
     fused = P > 1 and ops.fused_ring_step_supported(q)
     t = lambda x: None if x is None else x.transpose(1, 2)
@@ -147,7 +147,8 @@ def xdit_ring_flash_attn_forward(process_group, q, k, v, softmax_scale, dropout_
                 final = torch.empty((B, Sq, H, D), dtype=out_dtype, device=q.device)
             ops.attn_fwd_accumulate(t(q), t(key), t(value), t(out), lse.squeeze(-1).transpose(1, 2), first=step == 0,
                                     final_out=t(final), discard_acc_out=last, softmax_scale=softmax_scale,
-                                    k2=t(jk), v2=t(jv))
+                                    k2=t(jk), v2=t(jv), q_descale=q_descale, k_descale=k_descale,
+                                    v_descale=v_descale, out_dtype=out_dtype)
             continue
         block_out, block_lse = flash_attn_forward(
             q, key, value, dropout_p=dropout_p, softmax_scale=softmax_scale, causal=causal and step == 0,
