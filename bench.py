@@ -3,6 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
     python bench.py --model-shapes     (a table instead: see below)
+    python bench.py --ceiling-probes   (register-only probes of the matrix pipe, then the Flux step
+                                        on random and on constant inputs: what bounds the kernel)
 
 A "step" is one call of the joint-attention forward on the Flux-1024 shape
 (B=1, H=24, S=4608 = 512 text + 4096 image tokens, D=128, bf16, non-causal, BHSD-contiguous,
@@ -130,12 +132,19 @@ def with_rate(stat, flops, peak=None):
     return stat
 
 
-def series(dev, calls):
-    """Per-call HIP-event times (us) of the first `calls` Flux-1024 steps of this process."""
+def series(dev, calls, after_load=False):
+    """Per-call HIP-event times (us) of the first `calls` Flux-1024 steps of this process;
+    `after_load`: 150 bf16 matrix products of 8192^3 run first, so that the chip's power
+    management is already in its loaded state when the first step starts."""
     from xdit_amd import ops
     q, k, v = make_inputs(1, 24, 4608, 128, 1002, dev)
     out = torch.empty_like(q)
     lse = torch.empty(1, 24, 4608, dtype=torch.float32, device=dev)
+    if after_load:
+        a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        b = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        for _ in range(150):
+            torch.matmul(a, b)
     torch.cuda.synchronize()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(calls)]
     for a, b in ev:
@@ -144,6 +153,25 @@ def series(dev, calls):
         b.record()
     torch.cuda.synchronize()
     print(json.dumps([round(a.elapsed_time(b) * 1e3, 1) for a, b in ev]))
+
+
+def data_dependence(dev):
+    """The same launches on random and on constant inputs (steady state, per-call medians): the
+    instructions and the memory traffic are the same, the switching activity of the operands is not."""
+    from xdit_amd import ops
+    for name, (B, H, S) in (("Flux-1024 B=1 H=24 S=4608", (1, 24, 4608)), ("B=1 H=64 S=9216", (1, 64, 9216))):
+        q, k, v = make_inputs(B, H, S, 128, 1002, dev)
+        out = torch.empty_like(q)
+        fl = attn_flops(B, H, S, S, 128)
+        row = []
+        for label, (qq, kk, vv) in (("random q, k, v", (q, k, v)),
+                                    ("q = k = v = 0.5", tuple(torch.full_like(t, 0.5) for t in (q, k, v))),
+                                    ("only k constant", (q, torch.full_like(k, 0.5), v)),
+                                    ("only v constant", (q, k, torch.full_like(v, 0.5))),
+                                    ("only q constant", (torch.full_like(q, 0.5), k, v))):
+            st = time_each(lambda: ops.attn_fwd(qq, kk, vv, out=out), 100, 100)
+            row.append("%s %.1f us = %.0f TFLOP/s" % (label, st["ms"] * 1e3, fl / st["ms"] / 1e9))
+        print("data dependence, %s bf16: %s" % (name, " | ".join(row)), flush=True)
 
 
 def attn_flops(B, H, Sq, Sk, D):
@@ -262,6 +290,11 @@ def main():
                     help="print a table of the reference's model shapes against torch's GPU flash attention, and exit")
     ap.add_argument("--series", type=int, default=0,
                     help="print the per-call HIP-event times (us) of the first N Flux-1024 steps of this process, and exit")
+    ap.add_argument("--series-after-load", action="store_true",
+                    help="with --series: run 150 large bf16 matrix products first (the chip is then already under load)")
+    ap.add_argument("--ceiling-probes", action="store_true",
+                    help="run xdit_amd/csrc/build/mfma_ceiling (MFMA rate on constant and random operands, per-XCD times, "
+                         "MFMA/VALU co-issue), then time the Flux step on random and on constant inputs, and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof byte counters)")
     args = ap.parse_args()
@@ -269,6 +302,15 @@ def main():
         print("bench.py: this build runs on ONE GPU only (no collectives / sharding code); --gpus %d is not supported" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
+    if args.ceiling_probes:  # the probe program runs as a child before this process touches the GPU
+        import subprocess
+        exe = os.path.join(ROOT, "xdit_amd", "csrc", "build", "mfma_ceiling")
+        r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+        sys.stdout.write(r.stdout)
+        sys.stdout.flush()
+        if r.returncode != 0:
+            print("bench.py: %s exited with %d: %s" % (exe, r.returncode, r.stderr[-300:]), file=sys.stderr)
+            sys.exit(1)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
@@ -281,7 +323,10 @@ def main():
         model_shapes(dev)
         return
     if args.series:
-        series(dev, args.series)
+        series(dev, args.series, args.series_after_load)
+        return
+    if args.ceiling_probes:
+        data_dependence(dev)
         return
     B, H, S, D = 1, 24, 4608, 128
     q, k, v = make_inputs(B, H, S, D, 1002, dev)
