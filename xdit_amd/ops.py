@@ -5,6 +5,7 @@ BHSD-contiguous tensors and BSHD-contiguous tensors viewed as BHSD are consumed 
 PyTorch is used for device memory and the current stream only.
 """
 import ctypes
+import threading
 
 import torch
 
@@ -89,8 +90,9 @@ def _workspace(device, stream, nbytes):
 TUNING = {"rows_per_workgroup": 0, "cu_count": 0, "deterministic": 0}
 
 # Argument structs are filled once per call signature (shapes, strides, dtypes, options) and kept:
-# a later call with the same signature only patches the pointers and the stream.
-_PLANS = {}
+# a later call with the same signature only patches the pointers and the stream.  One set per
+# thread: the structs are patched in place, and the C call that reads them releases the GIL.
+_TLS = threading.local()
 _PLANS_MAX = 512
 
 
@@ -217,13 +219,14 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     key = (q.dtype, out_dtype, device, _sig(q), _sig(k), _sig(v), _sig(k2), _sig(v2), _sig(out), _sig(lse),
            k.dtype, v.dtype, float(softmax_scale), bool(causal), q_descale is not None, k_descale is not None,
            v_descale is not None, acc_sig, TUNING["rows_per_workgroup"], TUNING["cu_count"], bool(deterministic))
-    plan = _PLANS.get(key)
+    plans = _TLS.__dict__.setdefault("plans", {})
+    plan = plans.get(key)
     if plan is None:
         plan = _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, (q_descale, k_descale, v_descale),
                                 out_dtype, out, lse, _acc, deterministic)
-        if len(_PLANS) >= _PLANS_MAX:
-            _PLANS.clear()
-        _PLANS[key] = plan
+        if len(plans) >= _PLANS_MAX:
+            plans.clear()
+        plans[key] = plan
     else:
         for d in (q_descale, k_descale, v_descale):  # values the signature does not cover
             if d is not None and (d.dtype != torch.float32 or tuple(d.shape) != plan.shape[:2] or d.device != device):
@@ -472,18 +475,39 @@ def qk_prologue(x, weight=None, eps=1e-6, norm=None, rotary_emb=None, rope="inte
     return out
 
 
-def qk_prologue_batch(jobs):
-    """Up to 8 prologue jobs of one dtype on one device in ONE launch.  Each job is a dict of the
-    keyword arguments of `qk_prologue` (with `x`).  Returns the list of outputs."""
+def prologue_batch_args(jobs):
+    """The argument structs of up to 8 prologue jobs (dicts of the keyword arguments of
+    `qk_prologue`, with `x`) as one ctypes array, for `launch_prologue_batch`; the outputs are in
+    the jobs' `out` entries (created when missing).  The array keeps the tensors it points to alive
+    only through the caller's own references."""
     if not 1 <= len(jobs) <= 8:
         raise ValueError("a batch holds 1 to 8 jobs")
-    keep, outs = [], []
+    keep = []
     arr = (_lib.PrologueArgs * len(jobs))()
     for i, j in enumerate(jobs):
         a, out = _prologue_job(j["x"], j.get("weight"), j.get("eps", 1e-6), j.get("norm"), j.get("rotary_emb"),
                                j.get("rope", "interleaved"), j.get("rope_row0", 0), j.get("rope_rows"), j.get("out"), keep)
         arr[i] = a
-        outs.append(out)
-    with _on_device(jobs[0]["x"].device):
-        _lib.check(_lib.lib().xdit_qk_prologue_batch(arr, len(jobs)))
-    return outs
+        j["out"] = out
+    arr._keep = keep
+    return arr
+
+
+def launch_prologue_batch(arr, count, device):
+    """One launch of the first `count` jobs of an array from `prologue_batch_args` on the current
+    stream of `device` (pointers may have been patched since)."""
+    stream = _stream(device)
+    for i in range(count):
+        arr[i].stream = stream
+    with _on_device(device):
+        rc = _lib.lib().xdit_qk_prologue_batch(arr, count)
+    if rc != 0:
+        _lib.check(rc)
+
+
+def qk_prologue_batch(jobs):
+    """Up to 8 prologue jobs of one dtype on one device in ONE launch.  Each job is a dict of the
+    keyword arguments of `qk_prologue` (with `x`).  Returns the list of outputs."""
+    arr = prologue_batch_args(jobs)
+    launch_prologue_batch(arr, len(jobs), jobs[0]["x"].device)
+    return [j["out"] for j in jobs]

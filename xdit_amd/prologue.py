@@ -8,6 +8,8 @@ transformer_wan.py:99-122).  The functions here keep the call surfaces of the pi
 it in one pass and write straight into the BHSD tensor the attention kernel reads, text and image
 streams side by side (no torch.cat).
 """
+import threading
+
 import torch
 
 from . import ops
@@ -90,6 +92,9 @@ def norm_rope(x, weight=None, eps=1e-6, freqs_cis=None, sequence_dim=1, norm="he
     return out
 
 
+_TLS = threading.local()   # cached argument structs are patched in place: one set per thread
+
+
 def flux_joint_qkv(query, key, value, encoder_query, encoder_key, encoder_value, heads,
                    norm_q, norm_k, norm_added_q, norm_added_k, image_rotary_emb, eps=1e-6):
     """Lines 116-147 and 170-172 of xFuserFluxAttnProcessor.__call__ (transformer_flux.py): head
@@ -98,23 +103,53 @@ def flux_joint_qkv(query, key, value, encoder_query, encoder_key, encoder_value,
     BHSD.  Inputs are the projection outputs [B,S_img,H*D] and [B,S_txt,H*D]; norm_* are the gain
     vectors (D entries, the tensors' dtype); image_rotary_emb = (cos, sin) of [S_txt+S_img, D].
     Returns q, k, v as BHSD-contiguous [B,H,S_txt+S_img,D]: ONE launch of six jobs, no intermediate tensor."""
+    srcs = (encoder_query, query, encoder_key, key, encoder_value, value)
+    gains = (norm_added_q, norm_q, norm_added_k, norm_k)
+    cos, sin = image_rotary_emb
+    # The six argument structs are filled once per call signature (shapes, strides, dtype, device)
+    # and kept; a later call only allocates the outputs and patches pointers and the stream.
+    sig = (heads, float(eps), query.dtype, query.device, cos.dtype, cos.shape, cos.stride(), sin.shape, sin.stride(),
+           tuple((t.shape, t.stride()) for t in srcs), tuple(None if g is None else (g.shape, g.stride(), g.dtype) for g in gains))
+    plans = _TLS.__dict__.setdefault("flux_plans", {})
+    plan = plans.get(sig)
     B, S_img, HD = query.shape
     S_txt = encoder_query.shape[1]
     D = HD // heads
-    cos, sin = image_rotary_emb
-    outs, jobs = [], []
-    for img, txt, w_img, w_txt, is_v in ((query, encoder_query, norm_q, norm_added_q, False),
-                                         (key, encoder_key, norm_k, norm_added_k, False),
-                                         (value, encoder_value, None, None, True)):
-        out = torch.empty((B, heads, S_txt + S_img, D), dtype=query.dtype, device=query.device)
-        for src, w, row0 in ((txt, w_txt, 0), (img, w_img, S_txt)):
-            xb = src.unflatten(-1, (heads, D)).transpose(1, 2)
-            n = xb.shape[2]
-            job = dict(x=xb, out=out[:, :, row0:row0 + n])
-            if not is_v:
-                job.update(weight=w, eps=eps, norm="head", rotary_emb=(cos[row0:row0 + n], sin[row0:row0 + n]),
-                           rope="interleaved")
-            jobs.append(job)
-        outs.append(out)
-    ops.qk_prologue_batch(jobs)
-    return tuple(outs)
+    outs = tuple(torch.empty((B, heads, S_txt + S_img, D), dtype=query.dtype, device=query.device) for _ in range(3))
+    if plan is None:
+        jobs = []
+        for t, (txt, img) in enumerate(((encoder_query, query), (encoder_key, key), (encoder_value, value))):
+            for src, w, row0 in ((txt, gains[2 * t] if t < 2 else None, 0), (img, gains[2 * t + 1] if t < 2 else None, S_txt)):
+                xb = src.unflatten(-1, (heads, D)).transpose(1, 2)
+                n = xb.shape[2]
+                job = dict(x=xb, out=outs[t][:, :, row0:row0 + n])
+                if t < 2:
+                    job.update(weight=w, eps=eps, norm="head", rotary_emb=(cos[row0:row0 + n], sin[row0:row0 + n]),
+                               rope="interleaved")
+                jobs.append(job)
+        arr = ops.prologue_batch_args(jobs)
+        # where each pointer of each job lies relative to the tensor it comes from
+        plan = (arr, [(arr[i].y - outs[i // 2].data_ptr(),
+                       arr[i].cos - cos.data_ptr() if arr[i].cos else None,
+                       arr[i].sin - sin.data_ptr() if arr[i].sin else None,
+                       gains[i] is not None and arr[i].weight == gains[i].data_ptr() if i < 4 else False) for i in range(6)])
+        if len(plans) >= 64:
+            plans.clear()
+        # a gain or table that had to be copied (not contiguous) cannot be patched by pointer: no plan then
+        if (cos.is_contiguous() and sin.is_contiguous()
+                and all(rec[3] or (i >= 4 or gains[i] is None) for i, rec in enumerate(plan[1]))):
+            plans[sig] = plan
+    else:
+        arr, recs = plan
+        cp, sp = cos.data_ptr(), sin.data_ptr()
+        for i in range(6):
+            a = arr[i]
+            y_off, c_off, s_off, has_w = recs[i]
+            a.x = srcs[i].data_ptr()
+            a.y = outs[i // 2].data_ptr() + y_off
+            if c_off is not None:
+                a.cos, a.sin = cp + c_off, sp + s_off
+            if has_w:
+                a.weight = gains[i].data_ptr()
+    ops.launch_prologue_batch(arr, 6, query.device)
+    return outs
