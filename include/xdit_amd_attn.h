@@ -151,7 +151,10 @@ int xdit_attn_fwd_noalloc(const xdit_attn_args* args);
  * c starts with range c and, with counter != 0, takes further ranges from a counter in the
  * workspace.  A query tile's partial results occupy at most `slots_per_tile` workspace slots.
  * bf16 / fp16 (head_dim up to 128; the geometry is that of head_dim 64 or 128, whichever is
- * the next one up) and fp8 (head_dim 128) only.  No counterpart in the reference.
+ * the next one up) and fp8 (head_dim 128).  fp32 (head_dim up to 128): whole tiles only, of 128
+ * rows with `kv_iterations` tiles of 32 keys, or, when those would leave more than a quarter of
+ * the compute units without a workgroup, of 64 rows with tiles of 64 keys.  No counterpart in the
+ * reference.
  */
 typedef struct {
   uint32_t struct_size;        /* = sizeof(xdit_launch_plan), set by the caller */

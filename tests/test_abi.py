@@ -335,6 +335,7 @@ def test_launch_plan_of_the_named_shapes():
     assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == _lib.XDIT_ERR_INVALID_ARG
     p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
     a.dtype = a.out_dtype = _lib.DTYPE_FP32
+    a.D = 136   # no kernel takes fp32 tensors of a head_dim above 128
     assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == _lib.XDIT_ERR_UNSUPPORTED
 
 
@@ -461,3 +462,19 @@ def test_every_tile_and_kv_iteration_is_covered_exactly_once(tmp_path):
     assert balanced > 100 and odd_balanced > 20 and streamed > 20
     out = subprocess.run([str(exe)], input="\n".join(lines) + "\n", capture_output=True, text=True)
     assert out.returncode == 0 and out.stdout.split("\n")[0] == "ok %d" % len(lines) and "merge map ok" in out.stdout, out.stdout[-400:]
+
+
+def test_launch_plan_of_the_fp32_kernel():
+    """fp32 problems run one workgroup per query tile: 128-row tiles with 32-key KV tiles, or
+    64-row tiles with 64-key KV tiles when the 128-row tiles would fill less than three quarters
+    of the compute units the launch is planned for."""
+    p = _plan(1, 16, 1024, 1024, dtype=_lib.DTYPE_FP32, D=72, cus=256)      # PixArt-512: 128 tiles of 128 rows
+    assert (p.rows_per_workgroup, p.query_tiles, p.kv_iterations, p.workgroups, p.workspace_bytes, p.ranges) == (64, 256, 16, 256, 0, 0)
+    p = _plan(2, 16, 4096, 4096, dtype=_lib.DTYPE_FP32, D=72, cus=256)      # PixArt-1024: 1024 tiles
+    assert (p.rows_per_workgroup, p.query_tiles, p.kv_iterations, p.whole_tiles) == (128, 1024, 128, 1024)
+    p = _plan(1, 3, 8192, 100, Sk2=40, dtype=_lib.DTYPE_FP32, D=128, cus=256)  # 192 tiles: exactly three quarters
+    assert (p.rows_per_workgroup, p.kv_iterations) == (128, 4 + 2)
+    p = _plan(1, 3, 8192, 100, Sk2=40, dtype=_lib.DTYPE_FP32, D=128, cus=304)
+    assert (p.rows_per_workgroup, p.query_tiles, p.kv_iterations, p.workgroups) == (64, 384, 2 + 1, 384)
+    p = _plan(1, 1, 70, 10, dtype=_lib.DTYPE_FP32, D=8, cus=1)              # planned for one compute unit
+    assert (p.rows_per_workgroup, p.query_tiles, p.workgroups) == (128, 1, 8)

@@ -358,12 +358,26 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
   if (int rc0 = check_tuning(a)) return rc0;
   const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128;
   const bool b16 = mfma16_path(a);
-  if (!fp8 && !b16) return fail(XDIT_ERR_UNSUPPORTED, "no launch plan for this dtype / head_dim (generic kernel: one workgroup per 64 query rows)");
   xdit::AttnParams p, q;
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.cu_count = a->cu_count;
   p.deterministic = a->deterministic;
+  if (a->dtype == XDIT_DTYPE_FP32 && a->D > 0 && a->D % 8 == 0 && a->D <= 128) {
+    // the fp32 kernel: one workgroup per query tile, no shared last round, no workspace
+    const int rows = xdit::attn_fwd_f32_rows(p);
+    const int keys = rows == 64 ? 64 : 32;
+    const uint32_t size = out->struct_size;
+    std::memset(out, 0, sizeof(*out));
+    out->struct_size = size;
+    out->rows_per_workgroup = rows;
+    out->query_tiles = (int32_t)(a->B * a->H * ((a->Sq + rows - 1) / rows));
+    out->kv_iterations = (int32_t)((a->Sk + keys - 1) / keys + (a->Sk2 + keys - 1) / keys);
+    out->whole_tiles = out->query_tiles;
+    out->workgroups = (out->query_tiles + 7) / 8 * 8;
+    return XDIT_OK;
+  }
+  if (!fp8 && !b16) return fail(XDIT_ERR_UNSUPPORTED, "no launch plan for this dtype / head_dim");
   const int rows = rows_per_block_16(a);
   const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q);
   const uint32_t size = out->struct_size;

@@ -2,9 +2,11 @@
 // (tensors of a smaller head_dim, a multiple of 8, run on the next one up: see PAD below).
 //
 // Work decomposition
-//   workgroup = 256 threads = 4 wavefronts; it owns 128 query rows of one (batch, head);
-//   wavefront w owns rows [32w, 32w+32).  Keys/values stream through LDS in tiles of 64 keys,
-//   double buffered, filled by direct global->LDS loads (16 bytes per lane).
+//   workgroup = NW wavefronts (4, 8 or 12); a query tile is 32 NW rows of one (batch, head) and
+//   wavefront w owns rows [32w, 32w+32) of it.  Keys/values stream through LDS in tiles of 64
+//   keys, double buffered, filled by direct global->LDS loads (16 bytes per lane).  A workgroup
+//   is persistent: it walks the segments (whole query tiles, shares of shared ones) that
+//   WorkgroupWalk deals it.
 //
 // MFMA orientation (v_mfma_f32_32x32x16_{bf16,f16}; A is 32x16, B is 16x32, lane l holds row/col
 // l%32 and the 8 contraction elements 8*(l/32)..+7; the 32x32 result puts column l%32 and rows

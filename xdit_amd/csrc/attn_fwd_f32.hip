@@ -314,18 +314,21 @@ static hipError_t launch_d(const AttnParams& q, int d8, dim3 grid, hipStream_t s
 // (Smaller workgroups without the key split were measured and do not help: PixArt-512 fp32,
 // 16 x 1024 rows: 136 / 140 / 156 us at 128 / 64 / 32 rows, since the number of wavefronts, each
 // bound by its own chain of MFMAs, stays the same.)
+int attn_fwd_f32_rows(const AttnParams& p) {
+  const int64_t tiles128 = (int64_t)p.B * p.H * ((p.Sq + 127) / 128);
+  return tiles128 * 4 < (int64_t)resident_cus(p.cu_count) * 3 ? 64 : 128;
+}
+
 hipError_t launch_attn_fwd_f32(const AttnParams& p, int D, hipStream_t stream) {
   if (D <= 0 || D % 8 != 0 || D > 128) return hipErrorInvalidValue;
   AttnParams q = p;
-  const int64_t tiles128 = (int64_t)p.B * p.H * ((p.Sq + 127) / 128);
-  const int ks = tiles128 * 4 < (int64_t)resident_cus(p.cu_count) * 3 ? 2 : 1;
-  const int rows = 128 / ks;
+  const int rows = attn_fwd_f32_rows(p);
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
   dim3 grid(q.tiles_per_xcd * 8);
   const bool fused = p.acc_out != nullptr;
-  if (ks == 2) return fused ? f32path::launch_d<1, 2, true>(q, D / 8, grid, stream) : f32path::launch_d<1, 2, false>(q, D / 8, grid, stream);
+  if (rows == 64) return fused ? f32path::launch_d<1, 2, true>(q, D / 8, grid, stream) : f32path::launch_d<1, 2, false>(q, D / 8, grid, stream);
   return fused ? f32path::launch_d<1, 1, true>(q, D / 8, grid, stream) : f32path::launch_d<1, 1, false>(q, D / 8, grid, stream);
 }
 

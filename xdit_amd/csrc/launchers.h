@@ -82,6 +82,7 @@ size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block, Att
 hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream);
 size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan = nullptr);
 hipError_t launch_attn_fwd_f32(const AttnParams& p, int D, hipStream_t stream);  // fp32 tensors only
+int attn_fwd_f32_rows(const AttnParams& p);  // query rows per workgroup the fp32 launch takes: 128, or 64 (64-key tiles split between wavefront pairs)
 hipError_t launch_fp8_quant(const QuantParams& p, int in_dtype, hipStream_t stream);
 hipError_t launch_qk_prologue(const PrologueParams& p, int dtype, hipStream_t stream);
 hipError_t launch_qk_prologue_batch(const PrologueBatch& b, int dtype, hipStream_t stream);

@@ -272,7 +272,7 @@ def launch_plan(q, k, k2=None, deterministic=None):
     """How `attn_fwd(q, k, v, k2=..)` would be launched (a dict of the fields of xdit_launch_plan):
     rows per workgroup, query tiles, whole tiles, shared ranges and their length, claimers,
     whether ranges are handed out through the counter, workgroups, workspace bytes.  Host
-    arithmetic only; bf16 / fp16 (head_dim 64, 128) and fp8 (head_dim 128)."""
+    arithmetic only; bf16 / fp16 / fp32 (head_dim up to 128) and fp8 (head_dim 128)."""
     a = _lib.AttnArgs()
     a.struct_size = ctypes.sizeof(_lib.AttnArgs)
     a.dtype = _code(q.dtype)
