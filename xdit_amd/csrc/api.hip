@@ -58,13 +58,6 @@ int check_tensor(const char* name, const void* p, const xdit_strides& st, int es
   return 0;
 }
 
-// Query rows per workgroup of the 16-bit and fp8 kernels: 384, 256 or 128, i.e. 12, 8 or 4
-// wavefronts sharing each K/V tile.  Picks the shape with the shortest estimated critical path: KV iterations of the
-// busiest compute unit (whole rounds of resident workgroups, or the balanced launch's shared last
-// round plus its fixed cost) times the rows a compute unit works on per iteration, with a small
-// penalty for the shapes that share a tile between fewer wavefronts.  Measured on Flux-1024
-// (72 KV tiles: 384 rows wins through the balanced launch) and on its ring chunks (18 KV tiles:
-// 256 rows, 0.079 ms against 0.101 ms at 384).
 // head_dim the 16-bit MFMA kernel is built for that holds a tensor head_dim of D (64 or 128; the
 // kernel treats the columns the tensors do not have as zeros), 0 if there is none.
 int kernel_head_dim(int D) { return D <= 0 || D % 8 != 0 || D > 128 ? 0 : (D <= 64 ? 64 : 128); }
@@ -73,7 +66,19 @@ bool mfma16_path(const xdit_attn_args* a) {
   return (a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && kernel_head_dim(a->D) != 0;
 }
 
-int rows_per_block_16(const xdit_attn_args* a) {
+// Query rows per workgroup of the 16-bit and fp8 kernels: 384, 256 or 128, i.e. 12, 8 or 4
+// wavefronts sharing each K/V tile.  Picks the shape with the shortest estimated time:
+//   time = rate * (KV iterations of the busiest workgroup) * rows * (workgroups sharing its compute unit)
+//          + (segments of that workgroup) * (cost of a segment's prologue and epilogue)
+//          + (cost of the partial results and the combine pass, for a balanced launch).
+// `plain`: the launch will not be balanced (the ring step).
+// 16-bit kernels: the rate depends on the wavefronts a SIMD holds (one 4-wavefront workgroup on a
+// compute unit leaves every SIMD a single wavefront with nothing to overlap its softmax with: 1.5
+// to 1.8 times the time per row of 12 wavefronts).  Rates (ns per query row and KV tile), segment
+// and split costs (us) are fitted to a sweep of 94 problems (B*H 2..48, S 1024..16896 and the
+// model families' cross-attention and ring-chunk shapes, each forced to each shape): the choice is
+// the fastest shape or within 5 % of it on all but six of them (worst 9 %), 0.5 % off on average.
+int rows_per_block_16(const xdit_attn_args* a, bool plain = false) {
   const int D = kernel_head_dim(a->D);
   if (D == 0) return 128;
   if (a->rows_per_workgroup != 0) return a->rows_per_workgroup;  // validated by check_tuning
@@ -82,12 +87,13 @@ int rows_per_block_16(const xdit_attn_args* a) {
   const int64_t bh = (int64_t)a->B * a->H;
   const int64_t nt = (a->Sk + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile + (a->Sk2 + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile;
   static const int kRows[3] = {384, 256, 128};
-  // head_dim 64: 384 and 128 rows run at the same rate, 256 rows 5 % slower (B=1 H=48 S=17776:
-  // 4.21 / 4.41 / 4.15 ms at 384 / 256 / 128 rows; a 1063-key ring chunk of B=2 H=24 S=4250:
-  // 103 / 96 / 79 us), so the number of rounds decides
-  static const double kPenalty128[3] = {1.0, 1.06, 1.12};
-  static const double kPenalty64[3] = {1.0, 1.10, 1.0};
-  const double* kPenalty = D == 64 ? kPenalty64 : kPenalty128;
+  // 16-bit: {384 rows, 256 rows, 128 rows with two workgroups on the compute unit, 128 rows alone}
+  static const double kRate128[4] = {6.04, 7.15, 8.19, 11.33}, kRate64[4] = {3.98, 4.16, 4.72, 7.31};
+  const double* rate = D == 64 ? kRate64 : kRate128;
+  const double seg_us = D == 64 ? 0.54 : 4.77, split_us = D == 64 ? 11.75 : 17.46;
+  // fp8 (head_dim 128): penalties of 1.00 / 1.06 / 1.12 for 12 / 8 / 4 wavefronts sharing a tile and five
+  // iterations' worth per segment (Wan shard 7.39 / 7.92 / 7.99 ms, B=1 H=40 S=8192 744 / 769 / 782 us)
+  static const double kPenaltyFp8[3] = {1.0, 1.06, 1.12};
   int best = 128;
   double best_cost = 0;
   for (int i = 0; i < 3; i++) {
@@ -100,15 +106,22 @@ int rows_per_block_16(const xdit_attn_args* a) {
     std::memset(&q, 0, sizeof(q));
     q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
     q.deterministic = a->deterministic;
-    xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8);
-    // every segment costs a few iterations' worth of prologue and epilogue (about 13 us: 5
-    // iterations at head_dim 128, 9 at head_dim 64), the combine pass about as much again
-    const double ovh = D == 64 ? 9.0 : 5.0;
-    const double units = q.split_units ? (double)(q.split_full / slots) * (nt + ovh) + q.split_share + 2 * ovh
-                                       : (double)((tiles + slots - 1) / slots) * (nt + ovh);
+    if (!plain) xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8);
     int64_t sharing = (tiles + cus - 1) / cus;  // workgroups on the busiest compute unit at once
-    if (sharing > per_cu) sharing = per_cu;
-    const double cost = units * rows * (double)sharing * kPenalty[i];
+    if (sharing > per_cu || q.split_units) sharing = per_cu;
+    double cost;
+    if (fp8) {
+      const double ovh = 5.0;
+      const double units = q.split_units ? (double)(q.split_full / slots) * (nt + ovh) + q.split_share + 2 * ovh
+                                         : (double)((tiles + slots - 1) / slots) * (nt + ovh);
+      cost = units * rows * (double)sharing * kPenaltyFp8[i];
+    } else {
+      const int64_t rounds = q.split_units ? q.split_full / slots : (tiles + slots - 1) / slots;
+      const double units = (double)rounds * nt + (q.split_units ? q.split_share : 0);
+      const double segs = (double)rounds + (q.split_units ? 1 : 0);
+      const double r = rate[rows == 128 ? (sharing > 1 ? 2 : 3) : i];
+      cost = r * units * rows * (double)sharing * 1e-3 + seg_us * segs * (double)sharing + (q.split_units ? split_us : 0.0);
+    }
     if (i == 0 || cost < best_cost) { best = rows; best_cost = cost; }
   }
   return best;
@@ -270,11 +283,11 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   hipError_t e;
   if (mfma16_path(a)) {
     p.d_actual = a->D;
-    e = acc != nullptr ? xdit::launch_attn_fwd_16_ring(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a), stream)
+    e = acc != nullptr ? xdit::launch_attn_fwd_16_ring(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a, true), stream)
                        : xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a), stream);
   } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
     if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
-    e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, rows_per_block_16(a), stream);
+    e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, rows_per_block_16(a, acc != nullptr), stream);
   } else {
     if (a->D > 128) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d above 128 is not implemented", a->D);
     e = xdit::launch_attn_fwd_f32(p, a->D, stream);  // fp32 tensors: every 16-bit case went to the 16-bit kernel
