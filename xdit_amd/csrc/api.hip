@@ -69,15 +69,17 @@ bool mfma16_path(const xdit_attn_args* a) {
 // Query rows per workgroup of the 16-bit and fp8 kernels: 384, 256 or 128, i.e. 12, 8 or 4
 // wavefronts sharing each K/V tile.  Picks the shape with the shortest estimated time:
 //   time = rate * (KV iterations of the busiest workgroup) * rows * (workgroups sharing its compute unit)
-//          + (segments of that workgroup) * (cost of a segment's prologue and epilogue)
+//          + (segments of that workgroup) * (workgroups sharing ...) * (exposed cost of a segment's prologue and epilogue)
 //          + (cost of the partial results and the combine pass, for a balanced launch).
 // `plain`: the launch will not be balanced (the ring step).
-// 16-bit kernels: the rate depends on the wavefronts a SIMD holds (one 4-wavefront workgroup on a
-// compute unit leaves every SIMD a single wavefront with nothing to overlap its softmax with: 1.5
-// to 1.8 times the time per row of 12 wavefronts).  Rates (ns per query row and KV tile), segment
-// and split costs (us) are fitted to a sweep of 94 problems (B*H 2..48, S 1024..16896 and the
-// model families' cross-attention and ring-chunk shapes, each forced to each shape): the choice is
-// the fastest shape or within 5 % of it on all but six of them (worst 9 %), 0.5 % off on average.
+// 16-bit kernels: rate and segment cost depend on what a compute unit holds.  One 4-wavefront
+// workgroup leaves every SIMD a single wavefront with nothing to overlap its softmax with (1.5 to
+// 1.8 times the time per row of 12 wavefronts); two of them hide each other's prologue and
+// epilogue, which a lone 8- or 12-wavefront workgroup exposes in full (what decides
+// cross-attention on a few dozen keys).  The nine constants per head_dim (ns per query row and
+// KV tile; us) are fitted to the three shapes' times on 289 problems: B*H 1..48, S 1024..20000,
+// head_dim 64..128, self-attention, ring chunks and cross-attention on 77..2304 keys.  There the
+// choice is 0.8 % slower than the fastest shape on average (worst 11 %).
 int rows_per_block_16(const xdit_attn_args* a, bool plain = false) {
   const int D = kernel_head_dim(a->D);
   if (D == 0) return 128;
@@ -88,9 +90,11 @@ int rows_per_block_16(const xdit_attn_args* a, bool plain = false) {
   const int64_t nt = (a->Sk + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile + (a->Sk2 + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile;
   static const int kRows[3] = {384, 256, 128};
   // 16-bit: {384 rows, 256 rows, 128 rows with two workgroups on the compute unit, 128 rows alone}
-  static const double kRate128[4] = {6.04, 7.15, 8.19, 11.33}, kRate64[4] = {3.98, 4.16, 4.72, 7.31};
+  static const double kRate128[4] = {4.84, 5.34, 6.48, 8.95}, kRate64[4] = {4.03, 4.08, 4.57, 6.19};
+  static const double kSeg128[4] = {8.71, 8.69, 1.41, 6.65}, kSeg64[4] = {3.56, 1.82, 0.36, 2.44};
   const double* rate = D == 64 ? kRate64 : kRate128;
-  const double seg_us = D == 64 ? 0.54 : 4.77, split_us = D == 64 ? 11.75 : 17.46;
+  const double* seg_us = D == 64 ? kSeg64 : kSeg128;
+  const double split_us = D == 64 ? 12.4 : 14.6;
   // fp8 (head_dim 128): penalties of 1.00 / 1.06 / 1.12 for 12 / 8 / 4 wavefronts sharing a tile and five
   // iterations' worth per segment (Wan shard 7.39 / 7.92 / 7.99 ms, B=1 H=40 S=8192 744 / 769 / 782 us)
   static const double kPenaltyFp8[3] = {1.0, 1.06, 1.12};
@@ -116,11 +120,13 @@ int rows_per_block_16(const xdit_attn_args* a, bool plain = false) {
                                          : (double)((tiles + slots - 1) / slots) * (nt + ovh);
       cost = units * rows * (double)sharing * kPenaltyFp8[i];
     } else {
-      const int64_t rounds = q.split_units ? q.split_full / slots : (tiles + slots - 1) / slots;
-      const double units = (double)rounds * nt + (q.split_units ? q.split_share : 0);
-      const double segs = (double)rounds + (q.split_units ? 1 : 0);
-      const double r = rate[rows == 128 ? (sharing > 1 ? 2 : 3) : i];
-      cost = r * units * rows * (double)sharing * 1e-3 + seg_us * segs * (double)sharing + (q.split_units ? split_us : 0.0);
+      // rounds of resident workgroups; a long plain launch streams its workgroups through the slots
+      const double rounds = q.split_units ? (double)(q.split_full / slots)
+                            : tiles <= 4 * (int64_t)slots ? (double)((tiles + slots - 1) / slots) : (double)tiles / slots + 0.5;
+      const double units = rounds * nt + (q.split_units ? q.split_share : 0);
+      const double segs = rounds + (q.split_units ? 1 : 0);
+      const int cls = rows == 128 ? (sharing > 1 ? 2 : 3) : i;
+      cost = rate[cls] * units * rows * (double)sharing * 1e-3 + seg_us[cls] * segs * (double)sharing + (q.split_units ? split_us : 0.0);
     }
     if (i == 0 || cost < best_cost) { best = rows; best_cost = cost; }
   }
