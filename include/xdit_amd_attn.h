@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define XDIT_ATTN_ABI_VERSION 6
+#define XDIT_ATTN_ABI_VERSION 7
 
 typedef enum {
   XDIT_OK = 0,
@@ -91,6 +91,10 @@ typedef struct {
                                   same pointer (with 0 here on the first call after allocating it):
                                   the counters the library keeps at its start are then still zero, and
                                   a small initialisation launch per call is spared.  0 is always valid */
+  int32_t balance;             /* 0 = the library decides from its time estimate whether a launch given a
+                                  workspace is balanced; 1 = never (plain launch); 2 = whenever the planner
+                                  offers a balanced plan (a tuning and testing aid, like rows_per_workgroup) */
+  int32_t reserved0;           /* must be 0 */
   const void* q;
   const void* k;
   const void* v;

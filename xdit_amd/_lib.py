@@ -9,7 +9,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libxdit_amd_attn.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 XDIT_OK = 0
 XDIT_ERR_INVALID_ARG = -1
@@ -40,6 +40,8 @@ class AttnArgs(ctypes.Structure):
         ("cu_count", ctypes.c_int32),
         ("deterministic", ctypes.c_int32),
         ("workspace_preserved", ctypes.c_int32),
+        ("balance", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
         ("q", ctypes.c_void_p),
         ("k", ctypes.c_void_p),
         ("v", ctypes.c_void_p),

@@ -66,69 +66,95 @@ bool mfma16_path(const xdit_attn_args* a) {
   return (a->dtype == XDIT_DTYPE_BF16 || a->dtype == XDIT_DTYPE_FP16) && kernel_head_dim(a->D) != 0;
 }
 
-// Query rows per workgroup of the 16-bit and fp8 kernels: 384, 256 or 128, i.e. 12, 8 or 4
-// wavefronts sharing each K/V tile.  Picks the shape with the shortest estimated time:
+// How the 16-bit and fp8 kernels are launched: query rows per workgroup (384, 256 or 128, i.e. 12,
+// 8 or 4 wavefronts sharing each K/V tile) and whether the last round of query tiles is balanced
+// over the compute units.  Of the up to six options the one with the shortest estimated time:
 //   time = rate * (KV iterations of the busiest workgroup) * rows * (workgroups sharing its compute unit)
 //          + (segments of that workgroup) * (workgroups sharing ...) * (exposed cost of a segment's prologue and epilogue)
-//          + (cost of the partial results and the combine pass, for a balanced launch).
-// `plain`: the launch will not be balanced (the ring step).
-// 16-bit kernels: rate and segment cost depend on what a compute unit holds.  One 4-wavefront
-// workgroup leaves every SIMD a single wavefront with nothing to overlap its softmax with (1.5 to
-// 1.8 times the time per row of 12 wavefronts); two of them hide each other's prologue and
-// epilogue, which a lone 8- or 12-wavefront workgroup exposes in full (what decides
-// cross-attention on a few dozen keys).  The nine constants per head_dim (ns per query row and
-// KV tile; us) are fitted to the three shapes' times on 289 problems: B*H 1..48, S 1024..20000,
-// head_dim 64..128, self-attention, ring chunks and cross-attention on 77..2304 keys.  There the
-// choice is 0.8 % slower than the fastest shape on average (worst 11 %).
-int rows_per_block_16(const xdit_attn_args* a, bool plain = false) {
+//          + for a balanced launch: its extra launches, and the partial results a compute unit writes and folds.
+// `plain`: the launch will not be balanced (the ring step, or a call without a workspace).
+// Rate and segment cost depend on what a compute unit holds.  One 4-wavefront workgroup leaves
+// every SIMD a single wavefront with nothing to overlap its softmax with (1.5 times the time per
+// row of 12 wavefronts); two of them hide each other's prologue and epilogue, which a lone 8- or
+// 12-wavefront workgroup exposes in full (what decides cross-attention on a few dozen keys).
+// Balancing pays wherever the tiles leave compute units idle in the last round (the best plain
+// launch is 21 % slower on average than the best of the six, up to 3.8 times on a few heads of
+// 1000 to 3000 tokens) and costs a few per cent where they do not.  The constants (ns per query
+// row and KV tile; us) are fitted to the times of every option, taken at settled clocks, on 413
+// 16-bit problems (B*H 1..48, S 1024..118800, head_dim 64..128; self-attention, ring chunks and
+// cross-attention on 77..4608 keys) and 207 fp8 problems.  There the choice is 1.0 % (head_dim
+// 128), 1.4 % (64) and 0.6 % (fp8) slower than the fastest option on average, 11 % at worst; on
+// 140 problems kept out of an earlier fit of the same form, 1.4 % and 2.0 %.
+struct LaunchChoice {
+  int rows;    // query rows per workgroup
+  int policy;  // AttnParams::split_policy: 1 plain launch, 2 balanced when the planner offers a plan
+};
+
+LaunchChoice choose_launch(const xdit_attn_args* a, bool plain = false) {
+  LaunchChoice best = {128, 1};
   const int D = kernel_head_dim(a->D);
-  if (D == 0) return 128;
-  if (a->rows_per_workgroup != 0) return a->rows_per_workgroup;  // validated by check_tuning
+  if (D == 0) return best;
   const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN;
   const int cus = xdit::resident_cus(a->cu_count);
   const int64_t bh = (int64_t)a->B * a->H;
   const int64_t nt = (a->Sk + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile + (a->Sk2 + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile;
   static const int kRows[3] = {384, 256, 128};
   // 16-bit: {384 rows, 256 rows, 128 rows with two workgroups on the compute unit, 128 rows alone}
-  static const double kRate128[4] = {4.84, 5.34, 6.48, 8.95}, kRate64[4] = {4.03, 4.08, 4.57, 6.19};
-  static const double kSeg128[4] = {8.71, 8.69, 1.41, 6.65}, kSeg64[4] = {3.56, 1.82, 0.36, 2.44};
+  static const double kRate128[4] = {5.65, 5.88, 6.93, 8.65}, kRate64[4] = {3.59, 3.56, 4.26, 6.17};
+  static const double kSeg128[4] = {8.25, 6.36, 2.05, 6.57}, kSeg64[4] = {2.57, 1.70, 0.42, 2.18};
   const double* rate = D == 64 ? kRate64 : kRate128;
   const double* seg_us = D == 64 ? kSeg64 : kSeg128;
-  const double split_us = D == 64 ? 12.4 : 14.6;
-  // fp8 (head_dim 128): penalties of 1.00 / 1.06 / 1.12 for 12 / 8 / 4 wavefronts sharing a tile and five
-  // iterations' worth per segment (Wan shard 7.39 / 7.92 / 7.99 ms, B=1 H=40 S=8192 744 / 769 / 782 us)
-  static const double kPenaltyFp8[3] = {1.0, 1.06, 1.12};
-  int best = 128;
-  double best_cost = 0;
+  // a balanced launch: its extra launches, and the partial results per compute unit (us per thousand rows)
+  const double split_us = D == 64 ? 1.73 : 3.72;
+  const double parts_us = D == 64 ? 18.12 : 28.82;
+  // fp8 (head_dim 128, up to three 4-wavefront workgroups per compute unit):
+  // {384 rows, 256 rows, 128 rows x 3 / x 2 / alone}
+  static const double kRateFp8[5] = {3.64, 4.01, 4.02, 4.99, 6.06}, kSegFp8[5] = {6.18, 5.00, 0.16, 1.62, 5.70};
+  const double split_fp8_us = 1.04, parts_fp8_us = 30.50;
+  double best_cost = -1;
   for (int i = 0; i < 3; i++) {
     const int rows = kRows[i];
+    if (a->rows_per_workgroup != 0 && a->rows_per_workgroup != rows) continue;  // validated by check_tuning
     const int per_cu = rows == 128 ? (fp8 ? 3 : 2) : 1;  // workgroups resident per compute unit
     const int64_t tiles = bh * ((a->Sq + rows - 1) / rows);
     if (tiles > 0x7fffffff) continue;
     const int slots = cus * per_cu;
-    xdit::AttnParams q;
-    std::memset(&q, 0, sizeof(q));
-    q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
-    q.deterministic = a->deterministic;
-    if (!plain) xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8);
-    int64_t sharing = (tiles + cus - 1) / cus;  // workgroups on the busiest compute unit at once
-    if (sharing > per_cu || q.split_units) sharing = per_cu;
-    double cost;
-    if (fp8) {
-      const double ovh = 5.0;
-      const double units = q.split_units ? (double)(q.split_full / slots) * (nt + ovh) + q.split_share + 2 * ovh
-                                         : (double)((tiles + slots - 1) / slots) * (nt + ovh);
-      cost = units * rows * (double)sharing * kPenaltyFp8[i];
-    } else {
+    for (int policy = 1; policy <= 2; policy++) {
+      if ((plain || a->balance == 1) && policy == 2) continue;
+      xdit::AttnParams q;
+      std::memset(&q, 0, sizeof(q));
+      q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
+      q.deterministic = a->deterministic;
+      q.split_policy = policy;
+      if (policy == 2) {
+        xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8);
+        if (q.split_units == 0) continue;  // no balanced plan for this shape
+      } else if (a->balance == 2 && !plain) {
+        // a balanced plan is to be taken when there is one: the plain launch only stands in without
+        xdit::AttnParams t = q;
+        t.split_policy = 2;
+        xdit::plan_split(t, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8);
+        if (t.split_units != 0) continue;
+      }
+      int64_t sharing = (tiles + cus - 1) / cus;  // workgroups on the busiest compute unit at once
+      if (sharing > per_cu || q.split_units) sharing = per_cu;
       // rounds of resident workgroups; a long plain launch streams its workgroups through the slots
       const double rounds = q.split_units ? (double)(q.split_full / slots)
                             : tiles <= 4 * (int64_t)slots ? (double)((tiles + slots - 1) / slots) : (double)tiles / slots + 0.5;
       const double units = rounds * nt + (q.split_units ? q.split_share : 0);
       const double segs = rounds + (q.split_units ? 1 : 0);
-      const int cls = rows == 128 ? (sharing > 1 ? 2 : 3) : i;
-      cost = rate[cls] * units * rows * (double)sharing * 1e-3 + seg_us[cls] * segs * (double)sharing + (q.split_units ? split_us : 0.0);
+      // partial results written and folded, in thousands of rows per compute unit
+      const double parts = q.split_units ? (double)(tiles - q.split_full) * q.split_pmax * rows / cus * 1e-3 : 0.0;
+      double cost;
+      if (fp8) {
+        const int cls = rows == 128 ? 5 - (int)sharing : i;
+        cost = kRateFp8[cls] * units * rows * (double)sharing * 1e-3 + kSegFp8[cls] * segs * (double)sharing + (q.split_units ? split_fp8_us + parts_fp8_us * parts : 0.0);
+      } else {
+        const int cls = rows == 128 ? (sharing > 1 ? 2 : 3) : i;
+        cost = rate[cls] * units * rows * (double)sharing * 1e-3 + seg_us[cls] * segs * (double)sharing + (q.split_units ? split_us + parts_us * parts : 0.0);
+      }
+      if (best_cost < 0 || cost < best_cost) { best.rows = rows; best.policy = policy; best_cost = cost; }
     }
-    if (i == 0 || cost < best_cost) { best = rows; best_cost = cost; }
   }
   return best;
 }
@@ -139,6 +165,8 @@ int check_tuning(const xdit_attn_args* a) {
   if (r != 0 && r != 128 && r != 256 && r != 384)
     return fail(XDIT_ERR_INVALID_ARG, "rows_per_workgroup %d must be 0, 128, 256 or 384", r);
   if (a->cu_count < 0 || a->cu_count > 4096) return fail(XDIT_ERR_INVALID_ARG, "cu_count %d must be between 0 and 4096", a->cu_count);
+  if (a->balance < 0 || a->balance > 2) return fail(XDIT_ERR_INVALID_ARG, "balance %d must be 0, 1 or 2", a->balance);
+  if (a->reserved0 != 0) return fail(XDIT_ERR_INVALID_ARG, "reserved0 must be 0");
   return 0;
 }
 
@@ -289,11 +317,15 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   hipError_t e;
   if (mfma16_path(a)) {
     p.d_actual = a->D;
-    e = acc != nullptr ? xdit::launch_attn_fwd_16_ring(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a, true), stream)
-                       : xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), rows_per_block_16(a), stream);
+    const LaunchChoice c = choose_launch(a, acc != nullptr || p.ws_out == nullptr);  // no workspace: the shape that suits a plain launch
+    p.split_policy = c.policy;
+    e = acc != nullptr ? xdit::launch_attn_fwd_16_ring(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), c.rows, stream)
+                       : xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), c.rows, stream);
   } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
     if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
-    e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, rows_per_block_16(a, acc != nullptr), stream);
+    const LaunchChoice c = choose_launch(a, acc != nullptr || p.ws_out == nullptr);
+    p.split_policy = c.policy;
+    e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, c.rows, stream);
   } else {
     if (a->D > 128) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d above 128 is not implemented", a->D);
     e = xdit::launch_attn_fwd_f32(p, a->D, stream);  // fp32 tensors: every 16-bit case went to the 16-bit kernel
@@ -358,9 +390,11 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.cu_count = a->cu_count;
   p.deterministic = a->deterministic;
-  if (a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128) return (int64_t)xdit::attn_fwd_fp8_workspace(p, rows_per_block_16(a));
-  if (!mfma16_path(a)) return 0;
-  return (int64_t)xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows_per_block_16(a));
+  if (!(a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128) && !mfma16_path(a)) return 0;
+  const LaunchChoice c = choose_launch(a);
+  p.split_policy = c.policy;
+  if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) return (int64_t)xdit::attn_fwd_fp8_workspace(p, c.rows);
+  return (int64_t)xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), c.rows);
 }
 
 int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
@@ -397,7 +431,9 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
     return XDIT_OK;
   }
   if (!fp8 && !b16) return fail(XDIT_ERR_UNSUPPORTED, "no launch plan for this dtype / head_dim");
-  const int rows = rows_per_block_16(a);
+  const LaunchChoice choice = choose_launch(a);
+  const int rows = choice.rows;
+  p.split_policy = choice.policy;
   const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q);
   const uint32_t size = out->struct_size;
   std::memset(out, 0, sizeof(*out));

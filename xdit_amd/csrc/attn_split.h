@@ -182,6 +182,9 @@ constexpr int kClaimsPerWorkgroup = 6;
 // for the next call on the same workspace, whatever its shape.
 constexpr size_t kCounterRegionBytes = 16384;
 
+// Fewest KV iterations of critical path a balanced launch must save to be offered at all.
+constexpr int kMinSaving = 12;
+
 // Iterations a member of a tile's group owns under streamed sharing (the loop needs two to start
 // drawing from the counter without waiting for it).
 constexpr int kStreamedOwn = 2;
@@ -207,11 +210,10 @@ static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int o
   if (rem == 0 || nt < 8) return 0;
   int share = (int)(((int64_t)rem * nt + slots - 1) / slots);  // iterations per workgroup
   if (share < 4) share = 4;
-  // Iterations of the critical path saved by filling the last round.  Idle CUs leave the busy
-  // ones more power (higher clock), so a partly filled round costs less than its length suggests;
-  // balance only when the saving clearly exceeds the cost of the extra prologues, the partial
-  // results and the combine pass (measured: about 10 iterations' worth).
-  if (nt - share < 48) return 0;
+  // Iterations of the critical path saved by filling the last round: a plan is offered when it
+  // saves at least kMinSaving of them; whether it is taken is the caller's decision (the time
+  // estimate of the C entry points compares it with the plain launch; split_policy 1 refuses it).
+  if (q.split_policy == 1 || nt - share < kMinSaving) return 0;
   // Few shared tiles with short shares: streamed sharing.  Every resident workgroup joins the
   // group of one shared tile; unless the caller asks for bit-reproducible results.
   if (streamed && !q.deterministic && share < 2 * kMinClaimLen && rem * 4 <= slots) {
@@ -228,11 +230,14 @@ static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int o
       return kCounterRegionBytes + split_parts_bytes(q, rows, D, out_bytes);
     }
   }
-  // Long shares are cut into several ranges that are claimed one after the other.
+  // Long shares are cut into several ranges that are claimed one after the other: as many per
+  // claimer as the minimum range length allows, up to `claims`, and of a length that gives every
+  // claimer that whole number of ranges (2.25 ranges per claimer would end with a quarter of the
+  // compute units running a third range alone).
   int len = share;
   if (claims > 1 && share >= 2 * kMinClaimLen) {
-    len = (share + claims - 1) / claims;
-    if (len < kMinClaimLen) len = kMinClaimLen;
+    const int per_claimer = share / kMinClaimLen < claims ? share / kMinClaimLen : claims;
+    len = (share + per_claimer - 1) / per_claimer;
   }
   const int units = (int)(((int64_t)rem * nt + len - 1) / len);
   const int claimers = units < slots ? units : slots;

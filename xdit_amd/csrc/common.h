@@ -67,6 +67,7 @@ struct AttnParams {
   int split_dyn;      // streamed sharing of the remaining tiles (see WorkgroupWalk)
   int split_s0;       // KV iterations every member of a tile's group owns before it draws from the counter
   int deterministic;  // fixed work geometry only (no streamed sharing): results reproducible bit for bit
+  int split_policy;   // 1: plain launch; 2: balance whenever the plan shortens the critical path by kMinSaving iterations
   // ring step (optional): the result is folded into an fp32 accumulator in the epilogue
   float* acc_out;     // (B,H,Sq,D) fp32 running output, nullptr: plain forward
   float* acc_lse;     // (B,H,Sq) fp32 running log-sum-exp

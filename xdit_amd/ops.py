@@ -86,8 +86,9 @@ def _workspace(device, stream, nbytes):
 
 # Launch tuning passed to the library with every attention call (fields of xdit_attn_args):
 # rows_per_workgroup 0 = the library's choice, else 128 / 256 / 384; cu_count 0 = the device's
-# compute units, else plan the launch as for that many.  Tests and sweeps set these.
-TUNING = {"rows_per_workgroup": 0, "cu_count": 0, "deterministic": 0}
+# compute units, else plan the launch as for that many; balance 0 = the library decides whether a
+# launch is balanced, 1 = never, 2 = whenever its planner offers a plan.  Tests and sweeps set these.
+TUNING = {"rows_per_workgroup": 0, "cu_count": 0, "deterministic": 0, "balance": 0}
 
 # Argument structs are filled once per call signature (shapes, strides, dtypes, options) and kept:
 # a later call with the same signature only patches the pointers and the stream.  One set per
@@ -121,6 +122,7 @@ def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype
     a.B, a.H, a.D = B, H, D
     a.rows_per_workgroup = int(TUNING["rows_per_workgroup"])
     a.cu_count = int(TUNING["cu_count"])
+    a.balance = int(TUNING["balance"])
     a.deterministic = 1 if deterministic else 0
     a.Sq, a.Sk = Sq, k.shape[2]
     a.softmax_scale = float(softmax_scale)
@@ -218,7 +220,7 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     acc_sig = None if _acc is None else (_sig(_acc[0]), _sig(_acc[1]), _acc[2], _acc[3])
     key = (q.dtype, out_dtype, device, _sig(q), _sig(k), _sig(v), _sig(k2), _sig(v2), _sig(out), _sig(lse),
            k.dtype, v.dtype, float(softmax_scale), bool(causal), q_descale is not None, k_descale is not None,
-           v_descale is not None, acc_sig, TUNING["rows_per_workgroup"], TUNING["cu_count"], bool(deterministic))
+           v_descale is not None, acc_sig, TUNING["rows_per_workgroup"], TUNING["cu_count"], TUNING["balance"], bool(deterministic))
     plans = _TLS.__dict__.setdefault("plans", {})
     plan = plans.get(key)
     if plan is None:
@@ -282,6 +284,7 @@ def launch_plan(q, k, k2=None, deterministic=None):
     a.Sk2 = 0 if k2 is None else k2.shape[2]
     a.rows_per_workgroup = int(TUNING["rows_per_workgroup"])
     a.cu_count = int(TUNING["cu_count"])
+    a.balance = int(TUNING["balance"])
     a.deterministic = 1 if (TUNING["deterministic"] if deterministic is None else deterministic) else 0
     p = _lib.LaunchPlan()
     p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
