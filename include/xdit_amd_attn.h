@@ -135,7 +135,8 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* args);
  * the library (one copy per GPU, held until the process ends) instead of a workspace of the
  * caller; args->workspace is ignored.  Nothing is allocated or freed by the call.  A problem whose
  * xdit_attn_workspace_bytes exceeds the array is rejected with XDIT_ERR_INVALID_ARG (use
- * xdit_attn_fwd with a workspace then); Flux-1024 (B=1, H=24, S=4608, D=128) needs 28.75 MB.
+ * xdit_attn_fwd with a workspace then, or set args->balance = 1: the plain launch needs no
+ * scratch); Flux-1024 (B=1, H=24, S=4608, D=128) needs 28.75 MB.
  * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (two streams,
  * two threads) race on it and must be serialised by the caller; calls on one stream are ordered.
  * The array needs no clearing between calls (the range counter in it is reset by a kernel of each

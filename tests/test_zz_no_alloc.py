@@ -73,6 +73,11 @@ def test_noalloc_refuses_what_does_not_fit(gpu):
         ops.attn_fwd(q, k, k, out=out, lse=lse, noalloc=True)
     torch.cuda.synchronize()
     assert bool((out == 7.0).all())   # nothing was launched
+    # the same problem as a plain launch (the tuning field balance = 1) needs no scratch
+    ops.attn_fwd(q, k, k, out=out, lse=lse, noalloc=True, balance=False)
+    ref, ref_lse = ops.attn_fwd(q, k, k, balance=False)
+    assert torch.equal(out, ref) and torch.equal(lse, ref_lse)
+    out.fill_(7.0)
     # a plain launch (no shared last round) needs no scratch and is accepted at any size
     small_k = k[:, :, :64]
     ops.attn_fwd(q, small_k, small_k, out=out, lse=lse, noalloc=True)

@@ -343,7 +343,7 @@ int xdit_attn_fwd_noalloc(const xdit_attn_args* a) {
   if (need < 0) return (int)need;
   if (need > (int64_t)XDIT_ATTN_NOALLOC_SCRATCH_BYTES)
     return fail(XDIT_ERR_INVALID_ARG,
-                "this problem needs %lld bytes of scratch, xdit_attn_fwd_noalloc holds %lld: call xdit_attn_fwd with a workspace of the caller",
+                "this problem needs %lld bytes of scratch, xdit_attn_fwd_noalloc holds %lld: call xdit_attn_fwd with a workspace of the caller, or set balance = 1 (plain launch, no scratch)",
                 (long long)need, (long long)XDIT_ATTN_NOALLOC_SCRATCH_BYTES);
   xdit_attn_args b = *a;
   b.workspace = nullptr;

@@ -199,8 +199,9 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     default (the reference passes deterministic=False everywhere) a balanced launch may share
     the KV iterations of a query tile dynamically and results are reproducible to rounding.
     `noalloc=True` goes through the library's entry point that allocates nothing: the scratch is
-    a fixed buffer inside the library (problems that need more than it holds raise ValueError),
-    and `out` (and `lse` when `return_lse`) must be given.
+    a fixed buffer inside the library (problems that need more than it holds raise ValueError
+    unless `balance=False` asks for the plain launch), and `out` (and `lse` when `return_lse`)
+    must be given.
     """
     if (k2 is None) != (v2 is None):
         raise ValueError("k2 and v2 should be None or not None simultaneously.")
@@ -257,7 +258,10 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
             rc = L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r))
         elif noalloc:
             a.workspace, a.workspace_bytes = None, 0
+            if not balance:
+                a.balance = 1   # plain launch: no scratch at all, whatever the size
             rc = L.xdit_attn_fwd_noalloc(ctypes.byref(a))
+            a.balance = int(TUNING["balance"])
         else:
             if balance and plan.need > 0:
                 ws, preserved = _workspace(device, stream, plan.need)
