@@ -459,6 +459,39 @@ def test_fp8_small_vs_oracle(gpu, Sq, Sk):
     assert _err(o, ro) <= 6e-2 * max(1.0, ro.abs().max().item()) and _err(l, rl) <= 1e-3
 
 
+@pytest.mark.parametrize("balance", [1, 2])
+@pytest.mark.parametrize("rows", [128, 256, 384])
+@pytest.mark.parametrize("kind,D", [("bf16", 128), ("bf16", 64), ("fp16", 96), ("fp8", 128)])
+def test_every_launch_option_vs_oracle(gpu, monkeypatch, kind, D, rows, balance):
+    """The six ways a problem can be launched -- 128, 256 or 384 query rows per workgroup, as a plain
+    launch or with the last round balanced -- each forced through the tuning fields of
+    xdit_attn_args on a problem where all six exist (5 heads of 1000 rows on 1100 + 100 keys: no
+    workgroup shape fills the chip, so every query tile is shared), against the float64 oracle.
+    The default (whichever of the six the library's time estimate picks) is checked too."""
+    g = torch.Generator().manual_seed(D + rows + balance)
+    q, k, v, k2, v2 = (torch.randn(1, 5, n, D, generator=g) for n in (1000, 1100, 1100, 100, 100))
+    if kind == "fp8":
+        (q, qd), (kk, kd), (vv, vd) = (O.per_head_quant_ref(t) for t in (q, torch.cat([k, k2], 2), torch.cat([v, v2], 2)))
+        k, k2, v, v2 = kk[:, :, :1100], kk[:, :, 1100:], vv[:, :, :1100], vv[:, :, 1100:]
+        ro, rl = O.attn_fwd_ref(O.dequant(q, qd), O.dequant(kk, kd), O.dequant(vv, vd))
+        kw = dict(q_descale=qd.to(gpu), k_descale=kd.to(gpu), v_descale=vd.to(gpu))
+        tol = (6e-2, 1e-3)
+    else:
+        dtype = torch.bfloat16 if kind == "bf16" else torch.float16
+        q, k, v, k2, v2 = (t.to(dtype) for t in (q, k, v, k2, v2))
+        ro, rl = O.attn_fwd_ref(q, torch.cat([k, k2], 2), torch.cat([v, v2], 2))
+        kw, tol = {}, TOL[dtype]
+    dq, dk, dv, dk2, dv2 = (t.to(gpu) for t in (q, k, v, k2, v2))
+    for forced in (True, False):
+        monkeypatch.setitem(ops.TUNING, "rows_per_workgroup", rows if forced else 0)
+        monkeypatch.setitem(ops.TUNING, "balance", balance if forced else 0)
+        plan = ops.launch_plan(dq, dk, k2=dk2)
+        if forced:
+            assert plan["rows_per_workgroup"] == rows and (plan["ranges"] > 0) == (balance == 2), plan
+        o, l = ops.attn_fwd(dq, dk, dv, k2=dk2, v2=dv2, **kw)
+        assert _err(o, ro) <= tol[0] and _err(l, rl) <= tol[1], (forced, plan)
+
+
 # ---------------------------------------------------------------------------- merge
 @pytest.mark.parametrize("block_dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("layout", ["bhsd", "bshd"])
