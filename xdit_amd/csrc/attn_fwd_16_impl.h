@@ -297,6 +297,7 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
           constexpr int younger = (i_ + PD <= NR ? PD : NR - i_) - 1;
           lds_wait<younger>(kf[i_]);
           sacc[i_ / KSTEPS] = Mfma16<T>::mma(kf[i_], qf[i_ % KSTEPS], sacc[i_ / KSTEPS]);
+          if constexpr (i_ + PD >= NR && i_ + 1 < NR) __builtin_amdgcn_sched_barrier(0);  // issued before the next wait, not after the last one
           if constexpr (i_ + PD < NR) {
             constexpr int n = i_ + PD;
             lds_read_b128<(n / KSTEPS) * K_KB_STEP + (n % KSTEPS) * 32>(kf[n], kaddr);
@@ -369,6 +370,7 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
           lds_wait2<younger>(v0[i_], v1[i_]);
           s16x8 vv = __builtin_shufflevector(v0[i_], v1[i_], 0, 1, 2, 3, 4, 5, 6, 7);
           oacc[i_ % DBLOCKS] = Mfma16<T>::mma(__builtin_bit_cast(vec8, vv), pf[i_ / DBLOCKS], oacc[i_ % DBLOCKS]);
+          if constexpr (i_ + PD >= NM && i_ + 1 < NM) __builtin_amdgcn_sched_barrier(0);
           if constexpr (i_ + PD < NM) {
             constexpr int n = i_ + PD;
             constexpr int off = (n / DBLOCKS) * V_J_STEP + (n % DBLOCKS) * 64;
