@@ -283,10 +283,10 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
       {
         constexpr int PD = kPrefetch;   // K fragment reads in flight
         constexpr int NR = 2 * KSTEPS;  // reads (= MFMAs) of this product
-        vec8 kf[NR];
+        vec8 kf[NR];  // in MFMA order: contraction step i / 2 of key block i % 2, so that consecutive MFMAs share their Q fragment
         static_for<PD>([&](auto I) {
           constexpr int i_ = I;
-          lds_read_b128<(i_ / KSTEPS) * K_KB_STEP + (i_ % KSTEPS) * 32>(kf[i_], kaddr);
+          lds_read_b128<(i_ % 2) * K_KB_STEP + (i_ / 2) * 32>(kf[i_], kaddr);
         });
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
@@ -296,11 +296,11 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
           constexpr int i_ = I;
           constexpr int younger = (i_ + PD <= NR ? PD : NR - i_) - 1;
           lds_wait<younger>(kf[i_]);
-          sacc[i_ / KSTEPS] = Mfma16<T>::mma(kf[i_], qf[i_ % KSTEPS], sacc[i_ / KSTEPS]);
+          sacc[i_ % 2] = Mfma16<T>::mma(kf[i_], qf[i_ / 2], sacc[i_ % 2]);
           if constexpr (i_ + PD >= NR && i_ + 1 < NR) __builtin_amdgcn_sched_barrier(0);  // issued before the next wait, not after the last one
           if constexpr (i_ + PD < NR) {
             constexpr int n = i_ + PD;
-            lds_read_b128<(n / KSTEPS) * K_KB_STEP + (n % KSTEPS) * 32>(kf[n], kaddr);
+            lds_read_b128<(n % 2) * K_KB_STEP + (n / 2) * 32>(kf[n], kaddr);
           }
         });
       }
