@@ -205,7 +205,8 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
       const unsigned vaddr = vbase_off + buf * BUF_BYTES;
 
       // ---- S^T = K Q^T ---------------------------------------------------------------------
-      // Four MFMAs; MFMA m = 2 kb + ks takes the 32 bytes of its K row as two 16-byte reads.
+      // Four MFMAs; MFMA m = 2 ks + kb (consecutive ones share their Q fragment) takes the 32 bytes
+      // of its K row as two 16-byte reads.
       f32x16 sacc[2];
       {
         constexpr int PD = kPrefetch;  // MFMAs whose two reads are in flight
@@ -213,7 +214,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
         i32x4 klo[NM], khi[NM];
         static_for<PD>([&](auto I) {
           constexpr int m = I;
-          constexpr int off = (m / 2) * 4 * ROW_BYTES + (m % 2) * 64;
+          constexpr int off = (m % 2) * 4 * ROW_BYTES + (m / 2) * 64;
           lds_read_b128<off>(klo[m], kaddr);
           lds_read_b128<off + 16>(khi[m], kaddr);
         });
@@ -226,10 +227,10 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
           constexpr int younger = 2 * ((m + PD <= NM ? PD : NM - m) - 1);
           lds_wait2<younger>(klo[m], khi[m]);
           i32x8 kf = __builtin_shufflevector(klo[m], khi[m], 0, 1, 2, 3, 4, 5, 6, 7);
-          sacc[m / 2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[m % 2], sacc[m / 2], 0, 0, 0, 0, 0, 0);
+          sacc[m % 2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[m / 2], sacc[m % 2], 0, 0, 0, 0, 0, 0);
           if constexpr (m + PD < NM) {
             constexpr int n = m + PD;
-            constexpr int off = (n / 2) * 4 * ROW_BYTES + (n % 2) * 64;
+            constexpr int off = (n % 2) * 4 * ROW_BYTES + (n / 2) * 64;
             lds_read_b128<off>(klo[n], kaddr);
             lds_read_b128<off + 16>(khi[n], kaddr);
           }
