@@ -14,6 +14,11 @@
 //                followed by its share of the VALU work.  Constant and random operands, 8 and 12
 //                wavefronts per compute unit.  What the kernels add to this is LDS fragment reads,
 //                tile loads, barriers and waits.
+//   5. LDS reads    throughput per compute unit of the fragment reads of the 16-bit kernel, 12
+//                wavefronts reading and nothing else: ds_read_b128 and ds_read_b64_tr_b16 on
+//                contiguous addresses and on the kernel's K and V^T fragment address patterns.
+//   6. structure   the loop of the 16-bit kernel with its LDS reads and barrier (12 wavefronts of 32
+//                rows) against a pair structure (8 wavefronts of 64 rows) that reads 2.7 times less LDS.
 // Build: hipcc --offload-arch=gfx950 -O3 mfma_ceiling.hip -o mfma_ceiling ; run without arguments.
 #include <hip/hip_runtime.h>
 
@@ -238,6 +243,267 @@ static void loop_models(float* out) {
   CK(hipFree(in));
 }
 
+// ---- 5: LDS read throughput.  KIND 0: ds_read_b128, 16 B per lane contiguous; 1: ds_read_b64_tr_b16,
+// 8 B per lane contiguous; 2: ds_read_b128 on the K fragment pattern of the 16-bit kernel (head_dim
+// 128: key row r lives in piece r % 16 of 1040 B at slot r / 16 of 256 B; lane = (row, 16-byte half));
+// 3: ds_read_b64_tr_b16 on its V^T fragment pattern (pieces of 1088 B).
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+template <int KIND>
+__global__ __launch_bounds__(768) void lds_read_kernel(int* out, int iters) {
+  __shared__ __attribute__((aligned(16))) unsigned char smem[65536];
+  for (int i = threadIdx.x; i < 65536 / 4; i += 768) ((int*)smem)[i] = i;
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned addr = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  if (KIND == 0) addr += wave * 1024 + lane * 16;
+  else if (KIND == 1) addr += wave * 1024 + lane * 8;
+  else if (KIND == 2) addr += ((lane & 31) % 16) * 1040 + ((lane & 31) / 16) * 256 + (lane >> 5) * 16;
+  else addr += ((4 * (lane >> 5) + ((lane & 15) >> 2)) % 16) * 1088 + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  i32x4 acc = {0, 0, 0, 0};
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      if (KIND == 0 || KIND == 2) {
+        i32x4 v;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(j * 32));
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(v));
+        acc += v;
+      } else {
+        i32x2 v;
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(KIND == 3 ? (j & 3) * 64 + (j >> 2) * 8 * 1088 : j * 512));
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(v));
+        acc[0] += v[0];
+        acc[1] += v[1];
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)");
+  out[blockIdx.x * 768 + threadIdx.x] = acc[0] + acc[1] + acc[2] + acc[3];
+}
+template <int KIND>
+static void lds_read_rate(int* out, const char* name, int bytes_per_lane) {
+  const int iters = 20000;
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+  for (int w = 0; w < 3; w++) hipLaunchKernelGGL(lds_read_kernel<KIND>, dim3(kCUs), dim3(768), 0, 0, out, iters);
+  CK(hipEventRecord(e0));
+  hipLaunchKernelGGL(lds_read_kernel<KIND>, dim3(kCUs), dim3(768), 0, 0, out, iters);
+  CK(hipEventRecord(e1));
+  CK(hipEventSynchronize(e1));
+  float ms;
+  CK(hipEventElapsedTime(&ms, e0, e1));
+  const double bytes = 8.0 * iters * 12 * 64 * bytes_per_lane;  // per compute unit
+  printf("LDS reads, %s: %.0f bytes/ns per compute unit (%.0f bytes/clock at 2.4 GHz)\n", name, bytes / (ms * 1e6), bytes / (ms * 1e6) / 2.4);
+}
+
+// ---- 6: structure models WITH LDS traffic and barriers (values are meaningless, the instruction
+// streams are the kernels').  "present": 12 wavefronts x 32 query rows, every wavefront reads the
+// whole K tile (16 ds_read_b128) and V tile (32 ds_read_b64_tr_b16) of 64 keys, one barrier per
+// tile, the softmax of the attention kernel on its 32 values per lane.  "pair": 8 wavefronts x 64
+// query rows; the two wavefronts of a pair each compute S^T for 32 of the 64 keys, exchange their
+// P fragments through LDS (second barrier) and each accumulate 64 of the 128 head_dim columns, so
+// a wavefront reads 24 KiB of LDS per tile for 64 rows instead of 32 KiB for 32.
+typedef bf16x8 vec8;
+typedef __attribute__((ext_vector_type(4))) __bf16 vec4;
+typedef __attribute__((ext_vector_type(2))) __bf16 vec2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+#define LDS __attribute__((address_space(3)))
+__device__ __forceinline__ vec8 mma_in(s16x4 a, s16x4 b) { s16x8 v = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7); return __builtin_bit_cast(vec8, v); }
+__device__ __forceinline__ s16x4 read_tr(LDS unsigned char* p) { return __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS s16x4*)p); }
+__device__ __forceinline__ float max_of_halves(float x) { float y = __shfl_xor(x, 32); return fmaxf(x, y); }
+
+// softmax of one tile's 32 values per lane (as in the attention kernel): lazy max, exp2, row sum, bf16 P
+__device__ __forceinline__ void softmax32(const f32x16 (&s)[2], float& m_used, float& l, f32x16* o, int no, vec8 (&pf)[4], float c) {
+  float mx = s[0][0];
+#pragma unroll
+  for (int e = 1; e < 16; e++) mx = fmaxf(mx, s[0][e]);
+#pragma unroll
+  for (int e = 0; e < 16; e++) mx = fmaxf(mx, s[1][e]);
+  mx = max_of_halves(mx);
+  const float m_new = fmaxf(m_used, mx);
+  if (__builtin_amdgcn_ballot_w64((m_new - m_used) * c > 8.0f) != 0) {
+    const float alpha = __builtin_amdgcn_exp2f((m_used - m_new) * c);
+    m_used = m_new; l *= alpha;
+    for (int d = 0; d < no; d++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) o[d][e] *= alpha;
+  }
+  const float mc = m_used * c;
+#pragma unroll
+  for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][e], c, -mc));
+      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][e + 1], c, -mc));
+      l += p0 + p1;
+      f32x2 pp = {p0, p1};
+      vec2 pk = __builtin_convertvector(pp, vec2);
+      pf[2 * kb + (e >> 3)][e & 7] = pk[0];
+      pf[2 * kb + (e >> 3)][(e & 7) + 1] = pk[1];
+    }
+}
+
+constexpr int TILE = 32768;  // K 16 KiB + V 16 KiB per buffer
+
+__global__ __launch_bounds__(768) void present_structure_kernel(const vec8* in, float* out, int iters) {
+  extern __shared__ unsigned char smem_[];
+  LDS unsigned char* smem = (LDS unsigned char*)smem_;
+  const int lane = threadIdx.x & 63;
+  for (int i = threadIdx.x; i < 2 * TILE / 16; i += 768) ((LDS vec8*)smem)[i] = in[i & 4095];
+  vec8 qf[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) qf[k] = in[4096 + k * 768 + threadIdx.x];
+  f32x16 oacc[4] = {};
+  float m_used = -INFINITY, l = 0.f;
+  for (int it = 0; it < iters; it++) {
+    __syncthreads();
+    LDS unsigned char* kb_ = smem + (it & 1) * TILE;
+    LDS unsigned char* vb_ = kb_ + 16384;
+    f32x16 sacc[2] = {};
+    vec8 kf; s16x4 v0, v1;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      kf = *(LDS vec8*)(kb_ + i * 1024 + lane * 16);
+      sacc[i % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[i / 2], sacc[i % 2], 0, 0, 0);
+    }
+    vec8 pf[4];
+    softmax32(sacc, m_used, l, oacc, 4, pf, 0.1275f);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      v0 = read_tr(vb_ + i * 1024 + lane * 8);
+      v1 = read_tr(vb_ + i * 1024 + 512 + lane * 8);
+      oacc[i % 4] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(mma_in(v0, v1), pf[i / 4], oacc[i % 4], 0, 0, 0);
+    }
+  }
+  float s = l;
+  for (int d = 0; d < 4; d++) for (int e = 0; e < 16; e++) s += oacc[d][e];
+  out[blockIdx.x * 768 + threadIdx.x] = s;
+}
+
+__global__ __launch_bounds__(512) void pair_structure_kernel(const vec8* in, float* out, int iters) {
+  extern __shared__ unsigned char smem_[];
+  LDS unsigned char* smem = (LDS unsigned char*)smem_;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, role = wave & 1;
+  for (int i = threadIdx.x; i < 2 * TILE / 16; i += 512) ((LDS vec8*)smem)[i] = in[i & 4095];
+  LDS unsigned char* pbase = smem + 2 * TILE;  // 2 buffers x 8 wavefronts x 4 KiB of P
+  vec8 qf[2][8];
+#pragma unroll
+  for (int r = 0; r < 2; r++)
+#pragma unroll
+    for (int k = 0; k < 8; k++) qf[r][k] = in[4096 + (r * 8 + k) * 512 + threadIdx.x];
+  f32x16 oacc[4] = {};  // [db * 2 + rb]
+  float m_used[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+  for (int it = 0; it < iters; it++) {
+    __syncthreads();
+    LDS unsigned char* kb_ = smem + (it & 1) * TILE + role * 8192;           // this wavefront's 32 keys
+    LDS unsigned char* vb_ = smem + (it & 1) * TILE + 16384 + role * 8192;   // this wavefront's 64 head_dim columns
+    f32x16 sacc[2] = {};
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+      vec8 kf = *(LDS vec8*)(kb_ + ks * 1024 + lane * 16);
+      sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[0][ks], sacc[0], 0, 0, 0);
+      sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[1][ks], sacc[1], 0, 0, 0);
+    }
+    // per row block: 16 values per lane of this wavefront's 32 keys -> 2 P fragments each
+    vec8 pown[2][2];
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) {
+      float mx = sacc[rb][0];
+#pragma unroll
+      for (int e = 1; e < 16; e++) mx = fmaxf(mx, sacc[rb][e]);
+      mx = max_of_halves(mx);
+      const float m_new = fmaxf(m_used[rb], mx);
+      const float c = 0.1275f;
+      if (__builtin_amdgcn_ballot_w64((m_new - m_used[rb]) * c > 8.0f) != 0) {
+        const float alpha = __builtin_amdgcn_exp2f((m_used[rb] - m_new) * c);
+        m_used[rb] = m_new; l[rb] *= alpha;
+#pragma unroll
+        for (int e = 0; e < 16; e++) { oacc[rb][e] *= alpha; oacc[2 + rb][e] *= alpha; }
+      }
+      const float mc = m_used[rb] * c;
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[rb][e], c, -mc));
+        float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[rb][e + 1], c, -mc));
+        l[rb] += p0 + p1;
+        f32x2 pp = {p0, p1};
+        vec2 pk = __builtin_convertvector(pp, vec2);
+        pown[rb][e >> 3][e & 7] = pk[0];
+        pown[rb][e >> 3][(e & 7) + 1] = pk[1];
+      }
+    }
+    LDS unsigned char* pw = pbase + (it & 1) * 32768 + wave * 4096;
+    LDS unsigned char* pr = pbase + (it & 1) * 32768 + (wave ^ 1) * 4096;
+#pragma unroll
+    for (int j = 0; j < 4; j++) *(LDS vec8*)(pw + j * 1024 + lane * 16) = pown[j >> 1][j & 1];
+    __syncthreads();
+    vec8 pother[2][2];
+#pragma unroll
+    for (int j = 0; j < 4; j++) pother[j >> 1][j & 1] = *(LDS vec8*)(pr + j * 1024 + lane * 16);
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++)   // 16-key blocks: two of this wavefront's keys, two of the partner's
+#pragma unroll
+      for (int db = 0; db < 2; db++) {
+        const int i = kk * 2 + db;
+        s16x4 v0 = read_tr(vb_ + i * 1024 + lane * 8), v1 = read_tr(vb_ + i * 1024 + 512 + lane * 8);
+        const vec8 vf = mma_in(v0, v1);
+        oacc[db * 2 + 0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, kk < 2 ? pown[0][kk] : pother[0][kk - 2], oacc[db * 2 + 0], 0, 0, 0);
+        oacc[db * 2 + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, kk < 2 ? pown[1][kk] : pother[1][kk - 2], oacc[db * 2 + 1], 0, 0, 0);
+      }
+  }
+  float s = l[0] + l[1];
+  for (int d = 0; d < 4; d++) for (int e = 0; e < 16; e++) s += oacc[d][e];
+  out[blockIdx.x * 512 + threadIdx.x] = s;
+}
+
+
+template <typename K>
+static double structure_time(K kern, int threads, size_t lds, const vec8* in, float* out, int iters) {
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+  for (int w = 0; w < 8; w++) hipLaunchKernelGGL(kern, dim3(kCUs), dim3(threads), lds, 0, in, out, iters);
+  float best = 1e30f;
+  for (int r = 0; r < 5; r++) {
+    CK(hipEventRecord(e0));
+    hipLaunchKernelGGL(kern, dim3(kCUs), dim3(threads), lds, 0, in, out, iters);
+    CK(hipEventRecord(e1));
+    CK(hipEventSynchronize(e1));
+    float ms;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    if (ms < best) best = ms;
+  }
+  return best;
+}
+static void structure_models(float* out) {
+  const int iters = 4000;
+  const size_t n = 4096 + 16 * 768;
+  std::vector<unsigned short> h(n * 8);
+  vec8* d;
+  CK(hipMalloc(&d, n * 16));
+  CK(hipFuncSetAttribute((const void*)present_structure_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TILE));
+  CK(hipFuncSetAttribute((const void*)pair_structure_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TILE + 65536));
+  for (int mode = 0; mode < 2; mode++) {
+    srand(1);
+    for (auto& x : h) {
+      float f = mode ? (rand() / (float)RAND_MAX - 0.5f) * 2.0f : 0.0078125f;
+      unsigned u;
+      memcpy(&u, &f, 4);
+      x = (unsigned short)(u >> 16);
+    }
+    CK(hipMemcpy(d, h.data(), n * 16, hipMemcpyHostToDevice));
+    const double tc = structure_time(present_structure_kernel, 768, 2 * TILE, d, out, iters);
+    const double tp = structure_time(pair_structure_kernel, 512, 2 * TILE + 65536, d, out, iters);
+    printf("structure model with LDS reads and barriers, %s operands: present (12 x 32 rows) %.0f TFLOP/s | pair (8 x 64 rows) %.0f TFLOP/s of MFMA work\n",
+           mode ? "random" : "constant", kCUs * 12.0 * 32 * 32768.0 * iters / tc / 1e9, kCUs * 8.0 * 32 * 32768.0 * iters / tp / 1e9);
+  }
+  CK(hipFree(d));
+}
+
 int main() {
   const int G = kCUs, iters = 40000;
   std::vector<unsigned short> h(8 * 768 * 8);
@@ -283,6 +549,11 @@ int main() {
   coissue_table_fp8(out, 3);
   loop_models<false>(out);
   loop_models<true>(out);
+  lds_read_rate<0>((int*)out, "ds_read_b128, 16 bytes per lane contiguous", 16);
+  lds_read_rate<1>((int*)out, "ds_read_b64_tr_b16, 8 bytes per lane contiguous", 8);
+  lds_read_rate<2>((int*)out, "ds_read_b128 on the kernel's K fragment pattern", 16);
+  lds_read_rate<3>((int*)out, "ds_read_b64_tr_b16 on the kernel's V^T fragment pattern", 8);
+  structure_models(out);
   fflush(stdout);
   return 0;
 }
