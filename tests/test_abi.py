@@ -339,6 +339,59 @@ def test_launch_plan_of_the_named_shapes():
     assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == _lib.XDIT_ERR_UNSUPPORTED
 
 
+def test_launch_tuning_model_is_the_estimate_of_the_library():
+    """xdit_amd.launch_tuning (the tool that fits the constants of the library's launch choice) must
+    form the same terms as choose_launch in csrc/api.hip: with the constants read from that source
+    file, the cheapest of the six options under the Python model is the option the library picks,
+    for a few hundred random problems (host arithmetic only, 256 compute units)."""
+    import random
+    import re
+    from xdit_amd import launch_tuning as LT
+    src = open(os.path.join(os.path.dirname(_lib.__file__), "csrc", "api.hip")).read()
+    arr = lambda name: [float(v) for v in re.search(name + r"\[\d\] = \{([^}]*)\}", src).group(1).split(",")]
+    num = lambda pat: [float(v) for v in re.search(pat, src).groups()]
+    split64, split128 = num(r"split_us = D == 64 \? ([0-9.]+) : ([0-9.]+)")
+    parts64, parts128 = num(r"parts_us = D == 64 \? ([0-9.]+) : ([0-9.]+)")
+    split8, parts8 = num(r"split_fp8_us = ([0-9.]+), parts_fp8_us = ([0-9.]+)")
+    consts = {128: arr("kRate128") + arr("kSeg128") + [split128, parts128, 0.0],
+              64: arr("kRate64") + arr("kSeg64") + [split64, parts64, 0.0],
+              "fp8": arr("kRateFp8") + arr("kSegFp8") + [split8, parts8, 0.0]}
+    rng = random.Random(99)
+    checked = balanced = 0
+    for trial in range(300):
+        fp8 = rng.random() < 0.3
+        D = 128 if fp8 else rng.choice([128, 64, 96, 40])
+        shape = (1, rng.choice([1, 2, 3, 5, 8, 12, 24, 40]), rng.choice([1000, 2048, 4608, 9000, 20000, 75600]),
+                 rng.choice([77, 512, 1152, 4608, 20000]), D)
+        kw = dict(B=shape[0], H=shape[1], Sq=shape[2], Sk=shape[3], D=D, cu_count=256)
+        if fp8:
+            kw.update(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16)
+        def plan(**more):
+            a = _attn_args(**kw, **more)
+            p = _lib.LaunchPlan()
+            p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
+            assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == 0, _lib.last_error()
+            return p
+        auto = plan()
+        options = []
+        for rows in (384, 256, 128):          # the order in which the library tries them: the first of equals wins
+            for bal in (1, 2):
+                p = plan(rows_per_workgroup=rows, balance=bal)
+                if bal == 2 and p.ranges == 0:
+                    continue
+                o = {"rows": rows, "bal": bal, "tiles": p.query_tiles, "whole": p.whole_tiles, "ranges": p.ranges,
+                     "slots_per_tile": p.slots_per_tile}
+                f = LT.features(shape, o, fp8)
+                x = consts["fp8" if fp8 else (64 if D <= 64 else 128)]
+                options.append((sum(a_ * b_ for a_, b_ in zip(f, x)), (rows, bal)))
+        best = min(c for c, _ in options)
+        winners = [o for c, o in options if c <= best * (1 + 1e-12)]
+        assert (auto.rows_per_workgroup, 2 if auto.ranges else 1) == winners[0], (shape, fp8, options)
+        checked += 1
+        balanced += auto.ranges > 0
+    assert checked == 300 and 30 < balanced < 270
+
+
 WALK_HARNESS = r"""
 // Walks every workgroup of a planned launch with the code the kernels run (attn_walk.h) and
 // checks the coverage: stdin holds one launch per line.
