@@ -132,12 +132,15 @@ def with_rate(stat, flops, peak=None):
     return stat
 
 
-def series(dev, calls, after_load=False):
+def series(dev, calls, after_load=False, constant=False):
     """Per-call HIP-event times (us) of the first `calls` Flux-1024 steps of this process;
     `after_load`: 150 bf16 matrix products of 8192^3 run first, so that the chip's power
-    management is already in its loaded state when the first step starts."""
+    management is already in its loaded state when the first step starts; `constant`: q = k = v = 0.5
+    (same launches and traffic, far less switching activity in the matrix pipe)."""
     from xdit_amd import ops
     q, k, v = make_inputs(1, 24, 4608, 128, 1002, dev)
+    if constant:
+        q, k, v = (torch.full_like(t, 0.5) for t in (q, k, v))
     out = torch.empty_like(q)
     lse = torch.empty(1, 24, 4608, dtype=torch.float32, device=dev)
     if after_load:
@@ -292,6 +295,8 @@ def main():
                     help="print the per-call HIP-event times (us) of the first N Flux-1024 steps of this process, and exit")
     ap.add_argument("--series-after-load", action="store_true",
                     help="with --series: run 150 large bf16 matrix products first (the chip is then already under load)")
+    ap.add_argument("--series-constant", action="store_true",
+                    help="with --series: constant inputs (q = k = v = 0.5) instead of the random ones")
     ap.add_argument("--ceiling-probes", action="store_true",
                     help="run xdit_amd/csrc/build/mfma_ceiling (MFMA rate on constant and random operands, per-XCD times, "
                          "MFMA/VALU co-issue), then time the Flux step on random and on constant inputs, and exit")
@@ -323,7 +328,7 @@ def main():
         model_shapes(dev)
         return
     if args.series:
-        series(dev, args.series, args.series_after_load)
+        series(dev, args.series, args.series_after_load, args.series_constant)
         return
     if args.ceiling_probes:
         data_dependence(dev)
