@@ -17,6 +17,8 @@
 //   5. LDS reads    throughput per compute unit of the fragment reads of the 16-bit kernel, 12
 //                wavefronts reading and nothing else: ds_read_b128 and ds_read_b64_tr_b16 on
 //                contiguous addresses and on the kernel's K and V^T fragment address patterns.
+//   7. VALU rates   clocks per wavefront instruction and SIMD of the softmax's instructions (3 wavefronts
+//                per SIMD, four independent chains each).
 //   6. structure   the loop of the 16-bit kernel with its LDS reads and barrier (12 wavefronts of 32
 //                rows) against a pair structure (8 wavefronts of 64 rows) that reads 2.7 times less LDS.
 // Build: hipcc --offload-arch=gfx950 -O3 mfma_ceiling.hip -o mfma_ceiling ; run without arguments.
@@ -504,6 +506,38 @@ static void structure_models(float* out) {
   CK(hipFree(d));
 }
 
+// ---- 7: issue rate of the VALU instructions of the softmax (inline assembly, four independent chains)
+#define XDIT_REP8(X) X X X X X X X X
+template <int KIND>
+__global__ __launch_bounds__(768) void valu_rate_kernel(float* out, int iters) {
+  float a0 = threadIdx.x * 1e-3f, a1 = a0 + 1, a2 = a0 + 2, a3 = a0 + 3;
+  for (int i = 0; i < iters; i++) {
+    if (KIND == 0) { XDIT_REP8(asm volatile("v_exp_f32 %0, %0\n v_exp_f32 %1, %1\n v_exp_f32 %2, %2\n v_exp_f32 %3, %3" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));) }
+    if (KIND == 1) { XDIT_REP8(asm volatile("v_fma_f32 %0, %0, %1, %2\n v_fma_f32 %1, %1, %2, %3\n v_fma_f32 %2, %2, %3, %0\n v_fma_f32 %3, %3, %0, %1" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));) }
+    if (KIND == 2) { XDIT_REP8(asm volatile("v_add_f32 %0, %0, %1\n v_add_f32 %1, %1, %2\n v_add_f32 %2, %2, %3\n v_add_f32 %3, %3, %0" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));) }
+    if (KIND == 3) { XDIT_REP8(asm volatile("v_max3_f32 %0, %0, %1, %2\n v_max3_f32 %1, %1, %2, %3\n v_max3_f32 %2, %2, %3, %0\n v_max3_f32 %3, %3, %0, %1" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));) }
+    if (KIND == 4) { XDIT_REP8(asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2\n v_cvt_pk_bf16_f32 %1, %2, %3\n v_cvt_pk_bf16_f32 %2, %3, %0\n v_cvt_pk_bf16_f32 %3, %0, %1" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));) }
+    if (KIND == 5) { XDIT_REP8(asm volatile("v_cvt_pk_fp8_f32 %0, %1, %2\n v_cvt_pk_fp8_f32 %1, %2, %3\n v_cvt_pk_fp8_f32 %2, %3, %0\n v_cvt_pk_fp8_f32 %3, %0, %1" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));) }
+  }
+  out[blockIdx.x * 768 + threadIdx.x] = a0 + a1 + a2 + a3;
+}
+template <int KIND>
+static void valu_rate(float* out, const char* name) {
+  const int iters = 20000;
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+  for (int w = 0; w < 3; w++) hipLaunchKernelGGL(valu_rate_kernel<KIND>, dim3(kCUs), dim3(768), 0, 0, out, iters);
+  CK(hipEventRecord(e0));
+  hipLaunchKernelGGL(valu_rate_kernel<KIND>, dim3(kCUs), dim3(768), 0, 0, out, iters);
+  CK(hipEventRecord(e1));
+  CK(hipEventSynchronize(e1));
+  float ms;
+  CK(hipEventElapsedTime(&ms, e0, e1));
+  const double per_simd = 32.0 * iters * 3;  // wavefront instructions per SIMD
+  printf("VALU rate, %s: %.2f ns per wavefront instruction and SIMD (%.1f clocks at 2.4 GHz)\n", name, ms * 1e6 / per_simd, ms * 1e6 / per_simd * 2.4);
+}
+
 int main() {
   const int G = kCUs, iters = 40000;
   std::vector<unsigned short> h(8 * 768 * 8);
@@ -554,6 +588,12 @@ int main() {
   lds_read_rate<2>((int*)out, "ds_read_b128 on the kernel's K fragment pattern", 16);
   lds_read_rate<3>((int*)out, "ds_read_b64_tr_b16 on the kernel's V^T fragment pattern", 8);
   structure_models(out);
+  valu_rate<0>(out, "v_exp_f32");
+  valu_rate<1>(out, "v_fma_f32");
+  valu_rate<2>(out, "v_add_f32");
+  valu_rate<3>(out, "v_max3_f32");
+  valu_rate<4>(out, "v_cvt_pk_bf16_f32");
+  valu_rate<5>(out, "v_cvt_pk_fp8_f32");
   fflush(stdout);
   return 0;
 }
