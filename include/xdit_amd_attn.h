@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define XDIT_ATTN_ABI_VERSION 7
+#define XDIT_ATTN_ABI_VERSION 8
 
 typedef enum {
   XDIT_OK = 0,
@@ -81,16 +81,21 @@ typedef struct {
   float softmax_scale;         /* > 0 */
   int32_t cu_count;            /* 0 = plan the launch for the compute units of the current device;
                                   > 0 = for that many (tuning, testing, capacity planning) */
-  int32_t deterministic;       /* != 0: results reproducible bit for bit from call to call.  0 (the
-                                  value the reference passes for its `deterministic` option at every
-                                  call site): a balanced launch may hand KV iterations of a shared
-                                  query tile to whichever workgroup is free, so results are
-                                  reproducible only to rounding (the last bit of some outputs) */
+  int32_t streamed_sharing;    /* 0 (default): the work geometry of a launch is fixed, so results are
+                                  reproducible bit for bit from call to call, as those of the vendor
+                                  forwards this call replaces are (the reference's `deterministic`
+                                  option concerns its backward pass only: ring_flash_attn.py:190, :206,
+                                  :229).  != 0 opts in to a balanced launch that hands KV iterations of
+                                  a shared query tile to whichever workgroup is free: 1-2 % faster on
+                                  some shapes, results then reproducible only to rounding (the last
+                                  bit of some outputs) */
   int32_t workspace_preserved; /* != 0: the caller vouches that nothing but this library has written
                                   `workspace` since an earlier call of this library that was given the
-                                  same pointer (with 0 here on the first call after allocating it):
-                                  the counters the library keeps at its start are then still zero, and
-                                  a small initialisation launch per call is spared.  0 is always valid */
+                                  same pointer, returned XDIT_OK and had 0 here on the first call after
+                                  allocating the buffer (any such call will do: balanced or not, any
+                                  dtype; a call that is given a workspace of at least 16 KiB with 0 here
+                                  clears the counters at its start with a small launch).  The counters are
+                                  then still zero and that launch is spared.  0 is always valid */
   int32_t balance;             /* 0 = the library decides from its time estimate whether a launch given a
                                   workspace is balanced; 1 = never (plain launch); 2 = whenever the planner
                                   offers a balanced plan (a tuning and testing aid, like rows_per_workgroup) */
@@ -119,7 +124,8 @@ int xdit_attn_fwd(const xdit_attn_args* args);
  * Scratch bytes with which xdit_attn_fwd can balance this problem over the chip: when the number
  * of query tiles is not a multiple of what the GPU holds at once, the key/value range of the
  * tiles of the last, partly filled round is shared between workgroups, whose partial
- * (out, lse) pairs go through the workspace and are folded by a second small kernel.
+ * (out, lse) pairs go through the workspace and are folded by the workgroups themselves at their
+ * ends (tiles of up to 16 parts) or by a second small kernel.
  * Returns 0 when nothing would be gained, a negative xdit_status for invalid arguments
  * (pointers are not inspected).  Passing no or too small a workspace to xdit_attn_fwd is always
  * valid: the launch is then simply not balanced.  The workspace needs no initialisation and may
@@ -139,15 +145,20 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* args);
  * scratch); Flux-1024 (B=1, H=24, S=4608, D=128) needs 28.75 MB.
  * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (two streams,
  * two threads) race on it and must be serialised by the caller; calls on one stream are ordered.
- * The array needs no clearing between calls (the range counter in it is reset by a kernel of each
- * call).  No counterpart in the reference.
+ * The array needs no clearing between calls (the kernels of a call leave its counters at zero; after
+ * a call that failed a small launch clears them first).  It costs every GPU that the process uses
+ * the library on its XDIT_ATTN_NOALLOC_SCRATCH_BYTES of device memory from the moment the library is
+ * loaded, whether or not this entry point is ever called.  The first call on a device looks up the
+ * array's device address and sets a kernel attribute: make it outside any stream capture; later
+ * calls only launch kernels.  No counterpart in the reference.
  */
 #define XDIT_ATTN_NOALLOC_SCRATCH_BYTES (32 * 1024 * 1024)
 int xdit_attn_fwd_noalloc(const xdit_attn_args* args);
 
 /*
- * How xdit_attn_fwd would launch this problem when given the workspace it asks for (pointers of
- * `args` are not inspected): for tests, tuning and capacity planning.  The query rows are cut
+ * How xdit_attn_fwd (or, with plan->ring_step set, xdit_attn_fwd_accumulate) would launch this
+ * problem when given the workspace it asks for (pointers of `args` are not inspected): for tests,
+ * tuning and capacity planning.  The query rows are cut
  * into `query_tiles` tiles of `rows_per_workgroup` rows, each with `kv_iterations` tiles of 64
  * keys.  `whole_tiles` of them are run by one workgroup each; with ranges > 0 the KV iterations
  * of the other tiles, laid end to end, are cut into `ranges` ranges of `range_len` iterations
@@ -178,8 +189,14 @@ typedef struct {
   int32_t streamed;            /* != 0: streamed sharing instead of ranges: the `claimers` workgroups are dealt
                                   out over the shared tiles in contiguous groups; every member owns
                                   `range_len` KV iterations of its tile and draws the others one at a
-                                  time from the tile's counter (not with deterministic != 0) */
-  int32_t reserved0;
+                                  time from the tile's counter (only with streamed_sharing != 0) */
+  int32_t fold_in_kernel;      /* != 0: the parts of a shared tile are folded by the workgroups of the attention
+                                  kernel themselves (the ring step; tiles of at most 16 parts); 0: by a second
+                                  small kernel */
+  int32_t parts_first;         /* != 0: a claimer processes its range BEFORE its whole tile, and the workgroups
+                                  fold the shared tiles at their ends, a slice of rows each */
+  int32_t ring_step;           /* INPUT, set by the caller like struct_size: != 0 plans the launch of
+                                  xdit_attn_fwd_accumulate for these arguments, 0 that of xdit_attn_fwd */
 } xdit_launch_plan;
 
 int xdit_attn_launch_plan(const xdit_attn_args* args, xdit_launch_plan* plan);
@@ -232,7 +249,10 @@ int xdit_lse_merge(const xdit_merge_args* args);
  * (B,S,H,1) accumulator of the legacy ring maps without a copy).  bf16 / fp16 / fp32 inputs with
  * head_dim a multiple of 8 up to 128, fp8 inputs with head_dim 128; XDIT_ERR_UNSUPPORTED
  * otherwise (use the two calls).
- * args->workspace is not used.
+ * args->workspace (optional, as for xdit_attn_fwd: xdit_attn_workspace_bytes of the same arguments
+ * suffices) lets the launch be balanced: the parts of the shared query tiles are then folded and
+ * folded on into the accumulator by the attention kernel's own workgroups, and the result still
+ * equals xdit_attn_fwd with the same workspace and tuning fields + xdit_lse_merge bit for bit.
  * Replaces, per ring step: the kernel call at ring_flash_attn.py:123-134, update_out_and_lse at
  * :138 and, on the last step, the cast at :145.
  */

@@ -22,10 +22,10 @@ def gpu():
 
 @pytest.fixture(params=["deterministic", "streamed"])
 def sharing_mode(request, monkeypatch):
-    """Runs a GPU test twice: with the `deterministic` option of the attention call (fixed work
-    geometry, bit-reproducible results) and with the library's default, under which the KV
+    """Runs a GPU test twice: with the library's default (fixed work geometry, bit-reproducible
+    results) and with the `streamed_sharing` option of the attention call, under which the KV
     iterations of shared query tiles may go to whichever workgroup is free (results reproducible
     to rounding)."""
     from xdit_amd import ops
-    monkeypatch.setitem(ops.TUNING, "deterministic", 1 if request.param == "deterministic" else 0)
+    monkeypatch.setitem(ops.TUNING, "streamed", 0 if request.param == "deterministic" else 1)
     return request.param

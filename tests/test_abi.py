@@ -194,10 +194,10 @@ def test_workspace_query_needs_no_gpu():
     for s in ("q_stride", "k_stride", "v_stride", "out_stride"):
         setattr(a, s, _lib.Strides(24 * 4608 * 128, 4608 * 128, 128))
     need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
-    # streamed sharing: 8 workgroups per shared tile, one partial result each, plus the tiles' counters
-    assert need == 16384 + 32 * 8 * 384 * (128 * 2 + 4)   # 16 KiB of counters lead every workspace
-    a.deterministic = 1   # fixed ranges of 9 KV iterations: up to 72 / 9 + 1 parts per tile
-    assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) == 16384 + 32 * (72 // 9 + 1) * 384 * (128 * 2 + 4)
+    # fixed ranges of 9 KV iterations: up to 72 / 9 + 1 parts per tile; 16 KiB of counters lead every workspace
+    assert need == 16384 + 32 * (72 // 9 + 1) * 384 * (128 * 2 + 4)
+    a.streamed_sharing = 1   # 8 workgroups per shared tile, one partial result each
+    assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) == 16384 + 32 * 8 * 384 * (128 * 2 + 4)
     a.Sk = 64   # a single KV tile cannot be shared
     assert _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a)) == 0
 
@@ -240,8 +240,8 @@ def test_fused_ring_step_rejects_bad_arguments():
     assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "discard_acc_out" in _lib.last_error()
 
 
-def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128, rows=0, cus=0, det=True):
-    a = _attn_args(B=B, H=H, Sq=Sq, Sk=Sk, Sk2=Sk2, D=D, rows_per_workgroup=rows, cu_count=cus, deterministic=1 if det else 0)
+def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128, rows=0, cus=0, det=True, ring_step=False, balance=0):
+    a = _attn_args(B=B, H=H, Sq=Sq, Sk=Sk, Sk2=Sk2, D=D, rows_per_workgroup=rows, cu_count=cus, streamed_sharing=0 if det else 1, balance=balance)
     if dtype is not None:
         a.dtype = dtype
         a.out_dtype = _lib.DTYPE_BF16
@@ -249,9 +249,11 @@ def _plan(B, H, Sq, Sk, Sk2=0, dtype=None, D=128, rows=0, cus=0, det=True):
         a.k2 = a.v2 = 0x1000
     p = _lib.LaunchPlan()
     p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
+    p.ring_step = 1 if ring_step else 0
     rc = _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p))
     assert rc == 0, _lib.last_error()
-    assert p.workspace_bytes == _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
+    if not ring_step:
+        assert p.workspace_bytes == _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
     return p
 
 
@@ -339,59 +341,6 @@ def test_launch_plan_of_the_named_shapes():
     assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == _lib.XDIT_ERR_UNSUPPORTED
 
 
-def test_launch_tuning_model_is_the_estimate_of_the_library():
-    """xdit_amd.launch_tuning (the tool that fits the constants of the library's launch choice) must
-    form the same terms as choose_launch in csrc/api.hip: with the constants read from that source
-    file, the cheapest of the six options under the Python model is the option the library picks,
-    for a few hundred random problems (host arithmetic only, 256 compute units)."""
-    import random
-    import re
-    from xdit_amd import launch_tuning as LT
-    src = open(os.path.join(os.path.dirname(_lib.__file__), "csrc", "api.hip")).read()
-    arr = lambda name: [float(v) for v in re.search(name + r"\[\d\] = \{([^}]*)\}", src).group(1).split(",")]
-    num = lambda pat: [float(v) for v in re.search(pat, src).groups()]
-    split64, split128 = num(r"split_us = D == 64 \? ([0-9.]+) : ([0-9.]+)")
-    parts64, parts128 = num(r"parts_us = D == 64 \? ([0-9.]+) : ([0-9.]+)")
-    split8, parts8 = num(r"split_fp8_us = ([0-9.]+), parts_fp8_us = ([0-9.]+)")
-    consts = {128: arr("kRate128") + arr("kSeg128") + [split128, parts128, 0.0],
-              64: arr("kRate64") + arr("kSeg64") + [split64, parts64, 0.0],
-              "fp8": arr("kRateFp8") + arr("kSegFp8") + [split8, parts8, 0.0]}
-    rng = random.Random(99)
-    checked = balanced = 0
-    for trial in range(300):
-        fp8 = rng.random() < 0.3
-        D = 128 if fp8 else rng.choice([128, 64, 96, 40])
-        shape = (1, rng.choice([1, 2, 3, 5, 8, 12, 24, 40]), rng.choice([1000, 2048, 4608, 9000, 20000, 75600]),
-                 rng.choice([77, 512, 1152, 4608, 20000]), D)
-        kw = dict(B=shape[0], H=shape[1], Sq=shape[2], Sk=shape[3], D=D, cu_count=256)
-        if fp8:
-            kw.update(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16)
-        def plan(**more):
-            a = _attn_args(**kw, **more)
-            p = _lib.LaunchPlan()
-            p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
-            assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == 0, _lib.last_error()
-            return p
-        auto = plan()
-        options = []
-        for rows in (384, 256, 128):          # the order in which the library tries them: the first of equals wins
-            for bal in (1, 2):
-                p = plan(rows_per_workgroup=rows, balance=bal)
-                if bal == 2 and p.ranges == 0:
-                    continue
-                o = {"rows": rows, "bal": bal, "tiles": p.query_tiles, "whole": p.whole_tiles, "ranges": p.ranges,
-                     "slots_per_tile": p.slots_per_tile}
-                f = LT.features(shape, o, fp8)
-                x = consts["fp8" if fp8 else (64 if D <= 64 else 128)]
-                options.append((sum(a_ * b_ for a_, b_ in zip(f, x)), (rows, bal)))
-        best = min(c for c, _ in options)
-        winners = [o for c, o in options if c <= best * (1 + 1e-12)]
-        assert (auto.rows_per_workgroup, 2 if auto.ranges else 1) == winners[0], (shape, fp8, options)
-        checked += 1
-        balanced += auto.ranges > 0
-    assert checked == 300 and 30 < balanced < 270
-
-
 WALK_HARNESS = r"""
 // Walks every workgroup of a planned launch with the code the kernels run (attn_walk.h) and
 // checks the coverage: stdin holds one launch per line.
@@ -399,12 +348,32 @@ WALK_HARNESS = r"""
 #include <cstdlib>
 #include <vector>
 #include "attn_walk.h"
-struct Geom { int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers, split_dyn, split_s0; };
+struct Geom { int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers, split_dyn, split_s0, split_order; };
 int main() {
   Geom g; int nt, workgroups, counter, order; long line = 0;
-  while (scanf("%d %d %d %d %d %d %d %d %d %d %d %d %d %d", &g.total_tiles, &g.tiles_per_xcd, &g.split_full, &g.split_units, &g.split_len,
-               &g.split_pmax, &g.split_fuse0, &g.split_claimers, &nt, &workgroups, &counter, &order, &g.split_dyn, &g.split_s0) == 14) {
+  int fold;
+  while (scanf("%d %d %d %d %d %d %d %d %d %d %d %d %d %d %d %d", &g.total_tiles, &g.tiles_per_xcd, &g.split_full, &g.split_units, &g.split_len,
+               &g.split_pmax, &g.split_fuse0, &g.split_claimers, &nt, &workgroups, &counter, &order, &g.split_dyn, &g.split_s0, &g.split_order, &fold) == 16) {
     line++;
+    // fold duties (launches that fold inside the kernel): the word of every shared tile, which rows have been folded, and
+    // per workgroup the duties it has put off to its end (parts-first launches)
+    const int ROWS = 384;
+    std::vector<unsigned> word(g.total_tiles, 0u);
+    std::vector<int> folded((size_t)(fold ? (g.total_tiles - g.split_full) * ROWS : 0), 0);
+    std::vector<int> arrived(g.total_tiles, 0);
+    std::vector<std::vector<int>> duties(workgroups);
+    auto fold_now = [&](int r, unsigned mask, int n) {
+      if (mask && arrived[r] != n) { printf("line %ld: tile %d folded before its parts were there\n", line, r); exit(1); }
+      for (int j = 0; j < n; j++) if ((mask >> j) & 1u) { int r0, r1; xdit::fold_slice_rows(j, n, ROWS, r0, r1); for (int x = r0; x < r1; x++) folded[(size_t)r * ROWS + x]++; }
+    };
+    auto event = [&](int r, int j, int n, bool arrival, bool with_duty) {
+      const unsigned add = arrival ? xdit::fold_arrive_word(j, with_duty) : xdit::fold_duty_word(j);
+      const unsigned old = word[r];
+      word[r] += add;
+      if (arrival) arrived[r]++;
+      fold_now(r, arrival ? xdit::fold_after_arrival(old, j, with_duty, n) : xdit::fold_after_duty(old, j, n), n);
+      if (xdit::fold_last_event(old, add, n)) word[r] = 0u;
+    };
     std::vector<unsigned> tile_counter(g.total_tiles, 0u);
     std::vector<int> cover((size_t)g.total_tiles * nt, 0);
     const int rem = g.total_tiles - g.split_full;
@@ -417,7 +386,22 @@ int main() {
     bool any = true;
     auto step = [&](int w) {
       xdit::Segment s;
-      if (!walk[w].next(g, nt, s)) { live[w] = 0; return; }
+      if (!walk[w].next(g, nt, s)) {
+        live[w] = 0;
+        for (size_t d = 0; d + 2 < duties[w].size(); d += 3) event(duties[w][d], duties[w][d + 1], duties[w][d + 2], false, false);  // at the workgroup's end
+        if (g.split_order != 0) {  // the kernel works the duties out again from the workgroup's index: the same ones
+          std::vector<int> again;
+          const int u = w - g.split_fuse0, rem_iters = (g.total_tiles - g.split_full) * nt;
+          if (u >= 0 && u < g.split_units)
+            for (int lin = u * g.split_len, lin_end = lin + g.split_len < rem_iters ? lin + g.split_len : rem_iters; lin < lin_end;) {
+              const int r = lin / nt, it1 = lin_end - r * nt < nt ? lin_end - r * nt : nt;
+              again.push_back(r); again.push_back(u - (r * nt) / g.split_len); again.push_back(xdit::shared_tile_parts(g, nt, r));
+              lin = r * nt + it1;
+            }
+          if (again != duties[w]) { printf("line %ld: duties of workgroup %d\n", line, w); exit(1); }
+        }
+        return;
+      }
       if (s.tile < 0 || s.tile >= g.total_tiles || s.it0 < 0 || s.it1 > nt || s.it0 >= s.it1) { printf("line %ld: bad segment\n", line); exit(1); }
       for (int t = s.it0; t < s.it1; t++) cover[(size_t)s.tile * nt + t]++;
       if (s.dyn >= 0) {  // streamed sharing: draw the tile's other iterations one at a time, as the kernel does
@@ -434,6 +418,12 @@ int main() {
         const int r = s.tile - g.split_full;
         if (s.slot / g.split_pmax != r || s.slot % g.split_pmax >= xdit::shared_tile_parts(g, nt, r)) { printf("line %ld: slot outside its tile\n", line); exit(1); }
         slot_used[s.slot]++;
+        if (fold) {
+          const int n = xdit::shared_tile_parts(g, nt, r), j = (int)(s.slot % g.split_pmax);
+          if (n > xdit::kFoldMaxParts) { printf("line %ld: %d parts in a launch that folds in the kernel\n", line, n); exit(1); }
+          event(r, j, n, true, g.split_order == 0);
+          if (g.split_order != 0) { duties[w].push_back(r); duties[w].push_back(j); duties[w].push_back(n); }
+        }
       } else if (s.it0 != 0 || s.it1 != nt) { printf("line %ld: partial tile without a slot\n", line); exit(1); }
       if (walk[w].wants_claim(counter != 0 && !g.split_dyn)) walk[w].claimed(g, ticket++);
     };
@@ -452,6 +442,10 @@ int main() {
       }
     for (size_t i = 0; i < cover.size(); i++)
       if (cover[i] != 1) { printf("line %ld: tile %zu iteration %zu covered %d times\n", line, i / nt, i % nt, cover[i]); return 1; }
+    for (size_t i = 0; i < folded.size(); i++)
+      if (folded[i] != 1) { printf("line %ld: row %zu of shared tile %zu folded %d times\n", line, i % ROWS, i / ROWS, folded[i]); return 1; }
+    for (int r = 0; r < (fold ? rem : 0); r++)
+      if (word[r] != 0u) { printf("line %ld: fold word of tile %d left at %u\n", line, r, word[r]); return 1; }
     for (int r = 0; r < (g.split_units ? rem : 0); r++)
       for (int k = 0; k < g.split_pmax; k++)
         if (slot_used[(size_t)r * g.split_pmax + k] != (k < xdit::shared_tile_parts(g, nt, r) ? 1 : 0)) { printf("line %ld: slots of tile %d\n", line, r); return 1; }
@@ -486,14 +480,16 @@ def test_every_tile_and_kv_iteration_is_covered_exactly_once(tmp_path):
     (csrc/attn_walk.h compiled by g++): for compute-unit counts 1..304 (multiples of 8 or not) and
     random problems, every (query tile, KV iteration) is processed exactly once, every part of a
     shared tile lands in a slot of its own among those the fold reads, under three execution
-    orders of the workgroups.  Also the merge kernel's thread -> row map for head_dim 8..512."""
+    orders of the workgroups; and where the kernel folds the shared tiles itself, the fold-duty
+    protocol folds every row of every shared tile exactly once, never before all of the tile's
+    parts are there, and leaves the tiles' words at zero.  Also the merge kernel's thread -> row map for head_dim 8..512."""
     import random
     src = tmp_path / "walk.cpp"
     src.write_text(WALK_HARNESS)
     exe = tmp_path / "walk"
     subprocess.check_call(["g++", "-O1", "-std=c++17", "-I", os.path.join(ROOT, "xdit_amd", "csrc"), str(src), "-o", str(exe)])
     rng = random.Random(99)
-    lines, balanced, odd_balanced, streamed = [], 0, 0, 0
+    lines, balanced, odd_balanced, streamed, folds, parts_first = [], 0, 0, 0, 0, 0
     cases = [(cus, None) for cus in range(1, 305)] + [(rng.choice([0, 8, 64, 100, 252, 255, 256, 304]), i) for i in range(300)]
     for cus, extra in cases:
         fp8 = rng.random() < 0.25
@@ -502,17 +498,22 @@ def test_every_tile_and_kv_iteration_is_covered_exactly_once(tmp_path):
         Sq = rng.choice([rng.randint(1, 3000), rng.randint(3000, 40000), rng.randint(3000, 40000)])
         Sk = rng.choice([rng.randint(1, 600), rng.randint(3500, 12000), rng.randint(3500, 12000)])
         Sk2 = rng.choice([0, 0, rng.randint(1, 300)])
-        p = _plan(B, H, Sq, Sk, Sk2, dtype=_lib.DTYPE_FP8_E4M3FN if fp8 else None, rows=rows, cus=cus, det=rng.random() < 0.3)
+        ring_step = rng.random() < 0.5
+        p = _plan(B, H, Sq, Sk, Sk2, dtype=_lib.DTYPE_FP8_E4M3FN if fp8 else None, rows=rows, cus=cus, det=rng.random() < 0.3,
+                  ring_step=ring_step, balance=2 if ring_step else 0)
+        assert p.fold_in_kernel == (1 if ring_step and p.ranges else 0) and (ring_step or not p.parts_first)
         streamed += p.streamed
         fuse0 = p.first_claimer if p.ranges and p.first_claimer + p.claimers <= p.whole_tiles else 0x7fffffff
         full = p.whole_tiles if p.ranges else 0
         balanced += p.ranges > 0
         odd_balanced += p.ranges > 0 and full % 8 != 0
         for order in (0, 1, 2):
-            lines.append("%d %d %d %d %d %d %d %d %d %d %d %d %d %d" % (p.query_tiles, -(-p.query_tiles // 8), full, p.ranges, p.range_len,
-                                                                   p.slots_per_tile, fuse0, p.claimers, p.kv_iterations, p.workgroups, p.counter, order,
-                                                                   p.streamed, p.range_len if p.streamed else 0))
-    assert balanced > 100 and odd_balanced > 20 and streamed > 20
+            lines.append("%d %d %d %d %d %d %d %d %d %d %d %d %d %d %d %d" % (p.query_tiles, -(-p.query_tiles // 8), full, p.ranges, p.range_len,
+                                                                         p.slots_per_tile, fuse0, p.claimers, p.kv_iterations, p.workgroups, p.counter, order,
+                                                                         p.streamed, p.range_len if p.streamed else 0, p.parts_first, p.fold_in_kernel))
+        folds += p.fold_in_kernel
+        parts_first += p.parts_first
+    assert balanced > 100 and odd_balanced > 20 and streamed > 20 and folds > 50 and parts_first > 10 and balanced - folds > 50
     out = subprocess.run([str(exe)], input="\n".join(lines) + "\n", capture_output=True, text=True)
     assert out.returncode == 0 and out.stdout.split("\n")[0] == "ok %d" % len(lines) and "merge map ok" in out.stdout, out.stdout[-400:]
 

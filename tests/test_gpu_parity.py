@@ -28,7 +28,7 @@ def _err(a, b):
 
 
 def _same(a, b, mode):
-    """Two runs of one call: bit-identical with the deterministic option.  Otherwise the KV
+    """Two runs of one call: bit-identical by default.  Under streamed sharing the KV
     iterations of a shared query tile may be grouped into its partial results differently from
     run to run; the partial results are rounded to the output type before they are folded, so
     outputs of shared tiles then differ by about one unit in the last place of the LARGEST
@@ -368,7 +368,7 @@ def test_c2_flux1024_single_pass(gpu, sharing_mode, flux):
     assert _same(o, o4, sharing_mode) and (l - l4).abs().max().item() <= lse_tol
     assert _same(o, usp.USP(flux["q"], flux["k"], flux["v"]), sharing_mode)
     # whole query tiles do not depend on the sharing: the first 256 tiles of 384 rows are bit-identical
-    od, _ = ops.attn_fwd(flux["q"], flux["k"], flux["v"], deterministic=True)
+    od, _ = ops.attn_fwd(flux["q"], flux["k"], flux["v"], streamed=False)
     flat = lambda t: t.reshape(-1, 128)[: 256 * 384]
     assert torch.equal(flat(o), flat(od))
 
@@ -603,6 +603,32 @@ def test_smaller_head_dim_touches_only_its_columns(gpu, force_rows, rows, dtype,
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows", [128, 256, 384])
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 72), (torch.float16, 88)])
+def test_smaller_head_dim_in_a_balanced_launch(gpu, monkeypatch, rows, dtype, D):
+    """A head_dim below the kernel's own (72, 88 on the kernel built for 128) in a balanced launch,
+    where a workgroup runs several segments one after the other: between two segments the LDS
+    columns that no tile load writes are cleared again, which must wait until every wavefront is
+    done with its output staging block in the same memory (a workgroup that did not wait stored
+    zeros, or the neighbour's values, in some rows: a regression test).  Every row of three calls
+    against the plain launch (one workgroup per query tile) and probe rows against the oracle."""
+    monkeypatch.setitem(ops.TUNING, "rows_per_workgroup", rows)
+    monkeypatch.setitem(ops.TUNING, "balance", 2)
+    g = torch.Generator(device=gpu).manual_seed(D)
+    q, k, v = (torch.randn(1, 24, 4608, D, generator=g, device=gpu).to(dtype) for _ in range(3))
+    assert ops.launch_plan(q, k)["ranges"] > 0
+    plain_o, plain_l = ops.attn_fwd(q, k, v, balance=False)
+    for call in range(3):
+        out = torch.full_like(q, float("nan"))
+        lse = torch.full((1, 24, 4608), float("nan"), device=gpu)
+        ops.attn_fwd(q, k, v, out=out, lse=lse)
+        assert (out.float() - plain_o.float()).abs().max().item() <= 1e-2 and (lse - plain_l).abs().max().item() <= 1e-5, call
+    probe = torch.arange(0, 4608, 211)
+    ro, rl = O.attn_fwd_ref(q.cpu()[:, :, probe], k.cpu(), v.cpu())
+    assert _err(out[:, :, probe.to(gpu)], ro) <= 2e-2 and _err(lse[:, :, probe.to(gpu)], rl) <= 1e-3
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("seed", range(8))
 def test_random_problems_vs_oracle(gpu, monkeypatch, seed):
     """Random small problems over everything a call can vary: dtype, head_dim (every multiple of 8
@@ -761,6 +787,88 @@ def test_fused_ring_step_fp8_equals_forward_plus_merge(gpu, force_rows, out_dtyp
             oo, ol = (ro.to(out_dtype).double(), rl) if oo is None else O.merge_ref(oo, ol, ro.to(out_dtype), rl)
         assert torch.equal(fin, ref_fin)
         assert _err(acc_o, oo) <= 6e-2 and _err(acc_l, ol) <= 1e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,rows,H,Sq,Sk,parts_first,counter", [
+    ("bf16", 256, 3, 4608, 1152, 0, 0),      # every tile shared, parts of a tile end together: whoever completes it folds it
+    ("bf16", 256, 24, 4608, 4608, 1, 0),     # whole tiles too, one range per claimer: parts first, slices folded at the ends
+    ("bf16", 128, 24, 4608, 4608, 1, 0),
+    ("fp16", 256, 24, 4608, 3072, 1, 0),
+    ("bf16-d64", 256, 24, 4608, 4608, 1, 0),
+    ("bf16-d72", 128, 24, 4608, 4608, 1, 0),
+    ("bf16", 256, 12, 8192, 16384, 0, 1),    # long shares: ranges handed out through the counter
+    ("fp8", 256, 24, 4608, 4608, 1, 0),
+    ("fp8", 128, 24, 4608, 4608, 1, 0),
+])
+def test_balanced_fused_ring_step_equals_balanced_forward_plus_merge(gpu, monkeypatch, kind, rows, H, Sq, Sk, parts_first, counter):
+    """The ring step with a workspace: the shared query tiles of the last round go through the
+    workspace and are folded, and folded on into the accumulator, by the attention kernel's own
+    workgroups (fold duties).  Three steps (initialise; fold, with a joint KV segment; fold with
+    the final cast) must equal xdit_attn_fwd with the same launch geometry + xdit_lse_merge bit
+    for bit, twice in a row on the same workspace (its counters return to zero), and the oracle's
+    fold on probe rows."""
+    monkeypatch.setitem(ops.TUNING, "rows_per_workgroup", rows)
+    monkeypatch.setitem(ops.TUNING, "balance", 2)
+    monkeypatch.setitem(ops.TUNING, "streamed", 0)   # bit equality: the fixed work geometry on both sides
+    D = {"bf16-d64": 64, "bf16-d72": 72}.get(kind, 128)
+    dtype = torch.float16 if kind == "fp16" else torch.bfloat16
+    g = torch.Generator(device=gpu).manual_seed(H + Sk)
+    mk = lambda n: torch.randn(1, H, n, D, generator=g, device=gpu)
+    q = mk(Sq)
+    chunks = [(mk(Sk), mk(Sk)) for _ in range(3)]
+    jk, jv = mk(77), mk(77)
+    if kind == "fp8":
+        q_in, qs = ops.fp8_quant(q)
+        steps = []
+        for i, (k, v) in enumerate(chunks):
+            k8, j8, ks = ops.fp8_quant(k, x2=jk)
+            v8, w8, vs = ops.fp8_quant(v, x2=jv)
+            kw = dict(q_descale=qs, k_descale=ks, v_descale=vs, out_dtype=dtype)
+            if i == 1:
+                kw.update(k2=j8, v2=w8)
+            steps.append((k8, v8, kw))
+        ref_in = lambda t, s: O.dequant(t.cpu(), s.cpu())
+    else:
+        q_in = q.to(dtype)
+        steps = [(k.to(dtype), v.to(dtype), dict(k2=jk.to(dtype), v2=jv.to(dtype)) if i == 1 else {}) for i, (k, v) in enumerate(chunks)]
+    plan = ops.launch_plan(q_in, steps[0][0], ring_step=True)
+    assert plan["ranges"] > 0 and plan["fold_in_kernel"] == 1 and plan["parts_first"] == parts_first and plan["counter"] == counter, plan
+    assert ops.launch_plan(q_in, steps[0][0])["ranges"] == plan["ranges"]   # the plain forward is cut the same way
+    results = []
+    for repeat in range(2):
+        acc_o = torch.full((1, H, Sq, D), float("nan"), device=gpu)
+        acc_l = torch.full((1, H, Sq), float("nan"), device=gpu)
+        ref_o, ref_l = torch.empty_like(acc_o), torch.empty_like(acc_l)
+        fin = torch.empty(1, H, Sq, D, dtype=dtype, device=gpu)
+        ref_fin = torch.empty_like(fin)
+        for i, (k, v, kw) in enumerate(steps):
+            last = i + 1 == len(steps)
+            ops.attn_fwd_accumulate(q_in, k, v, acc_o, acc_l, first=i == 0, final_out=fin if last else None, **kw)
+            bo, bl = ops.attn_fwd(q_in, k, v, **kw)
+            ops.lse_merge(ref_o, ref_l, bo, bl, first=i == 0, final_out=ref_fin if last else None)
+            assert torch.equal(acc_o, ref_o) and torch.equal(acc_l, ref_l), (repeat, i)
+        assert torch.equal(fin, ref_fin)
+        results.append((acc_o, acc_l, fin))
+    assert all(torch.equal(a, b) for a, b in zip(*results))
+    # values: probe rows of the whole fold against the oracle
+    probe = torch.arange(0, Sq, 509)
+    oo = ol = None
+    for i, (k, v, kw) in enumerate(steps):
+        if kind == "fp8":
+            kd, vd = ref_in(k, kw["k_descale"]), ref_in(v, kw["v_descale"])
+            if i == 1:
+                kd, vd = torch.cat([kd, ref_in(kw["k2"], kw["k_descale"])], 2), torch.cat([vd, ref_in(kw["v2"], kw["v_descale"])], 2)
+            qd = ref_in(q_in, qs)
+        else:
+            kd, vd = k.cpu(), v.cpu()
+            if i == 1:
+                kd, vd = torch.cat([kd, kw["k2"].cpu()], 2), torch.cat([vd, kw["v2"].cpu()], 2)
+            qd = q_in.cpu()
+        ro, rl = O.attn_fwd_ref(qd[:, :, probe], kd, vd)
+        oo, ol = (ro.to(dtype).double(), rl) if oo is None else O.merge_ref(oo, ol, ro.to(dtype), rl)
+    tol = 6e-2 if kind == "fp8" else 2e-2
+    assert _err(results[0][0][:, :, probe.to(gpu)], oo) <= tol and _err(results[0][1][:, :, probe.to(gpu)], ol) <= 1e-3
 
 
 @pytest.mark.gpu

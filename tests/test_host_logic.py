@@ -209,31 +209,3 @@ def test_bench_refuses_more_than_one_gpu_and_lists_the_model_shapes():
         assert ops.fused_ring_step_supported(torch.empty(1, 1, 1, D, dtype=torch.bfloat16))
 
 
-def test_launch_tuning_sets_and_evaluation(tmp_path, capsys):
-    """The tuning tool's problem sets are what its documentation says, and `evaluate` reads a sweep
-    file and reports the loss of the library's choice (here a made-up file in which the option the
-    library picks is the fastest, so the loss is zero)."""
-    import ctypes
-    import json
-    from xdit_amd import _lib, launch_tuning as LT
-    assert len(LT.problem_set("grid", False)) == 136 and len(LT.problem_set("grid", True)) == 67
-    assert len(LT.problem_set("cross", False)) == 90 and len(LT.problem_set("long", True)) == 25
-    assert len(LT.problem_set("7", False)) == 70 and LT.problem_set("7", False) == LT.problem_set("7", False)
-    assert all(s[4] == 128 for s in LT.problem_set("9", True))
-    shape = (1, 24, 4608, 4608, 128)
-    a = _lib.AttnArgs()
-    a.struct_size = ctypes.sizeof(_lib.AttnArgs)
-    a.dtype = a.out_dtype = _lib.DTYPE_BF16
-    a.B, a.H, a.Sq, a.Sk, a.D = shape
-    a.softmax_scale, a.cu_count = 0.1, LT.CUS
-    p = _lib.LaunchPlan()
-    p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
-    assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == 0
-    chosen = (p.rows_per_workgroup, 2 if p.ranges else 1)
-    opts = [{"rows": r, "bal": b, "t": 100.0 if (r, b) == chosen else 150.0, "tiles": 1, "whole": 1, "ranges": 0, "len": 0,
-             "streamed": 0, "slots_per_tile": 0} for r in (128, 256, 384) for b in (1, 2)]
-    f = tmp_path / "sweep.jsonl"
-    f.write_text(json.dumps({"shape": shape, "opts": opts}) + "\n")
-    LT.evaluate([str(f)], False)
-    out = capsys.readouterr().out
-    assert "1 problems" in out and "0.0 % slower" in out and "50 % slower" in out

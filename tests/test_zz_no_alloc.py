@@ -16,9 +16,9 @@ LIMIT = 32 * 1024 * 1024
 
 @pytest.fixture(autouse=True)
 def fixed_geometry(monkeypatch):
-    """The comparison below is bit for bit, so both calls run with the `deterministic` option (under
-    the default, streamed sharing, two runs of ONE entry point already differ in last bits)."""
-    monkeypatch.setitem(ops.TUNING, "deterministic", 1)
+    """The comparison below is bit for bit, so both calls run with the default, fixed work geometry
+    (under streamed sharing two runs of ONE entry point already differ in last bits)."""
+    monkeypatch.setitem(ops.TUNING, "streamed", 0)
 
 
 def _pair(q, k, v, **kw):
@@ -49,11 +49,11 @@ def test_noalloc_entry_point_equals_attn_fwd(gpu):
     # the fp8 kernel shares the same array
     (q8, qd), (k8, kd), (v8, vd) = (ops.fp8_quant(t) for t in small)
     _pair(q8, k8, v8, q_descale=qd, k_descale=kd, v_descale=vd)
-    # the default sharing mode through the same entry point: equal to rounding
+    # streamed sharing through the same entry point: equal to rounding
     out = torch.empty_like(big[0])
     lse = torch.empty(1, 24, 4608, device=gpu)
-    ops.attn_fwd(*big, out=out, lse=lse, noalloc=True, deterministic=False)
-    assert ops.launch_plan(big[0], big[1], deterministic=False)["streamed"] == 1
+    ops.attn_fwd(*big, out=out, lse=lse, noalloc=True, streamed=True)
+    assert ops.launch_plan(big[0], big[1], streamed=True)["streamed"] == 1
     assert (out.float() - o1.float()).abs().max().item() <= 2.0 ** -7 * o1.float().abs().max().item()
     assert (lse - l1).abs().max().item() <= 1e-5
     # a sane value check on top of the equality: rows of the small problem against fp32 torch

@@ -9,7 +9,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libxdit_amd_attn.so")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 XDIT_OK = 0
 XDIT_ERR_INVALID_ARG = -1
@@ -38,7 +38,7 @@ class AttnArgs(ctypes.Structure):
         ("Sk2", ctypes.c_int64),
         ("softmax_scale", ctypes.c_float),
         ("cu_count", ctypes.c_int32),
-        ("deterministic", ctypes.c_int32),
+        ("streamed_sharing", ctypes.c_int32),
         ("workspace_preserved", ctypes.c_int32),
         ("balance", ctypes.c_int32),
         ("reserved0", ctypes.c_int32),
@@ -109,7 +109,9 @@ class LaunchPlan(ctypes.Structure):
         ("counter", ctypes.c_int32),
         ("workgroups", ctypes.c_int32),
         ("streamed", ctypes.c_int32),
-        ("reserved0", ctypes.c_int32),
+        ("fold_in_kernel", ctypes.c_int32),
+        ("parts_first", ctypes.c_int32),
+        ("ring_step", ctypes.c_int32),
     ]
 
 

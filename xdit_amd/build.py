@@ -30,10 +30,6 @@ def _hipcc():
     raise RuntimeError("hipcc not found")
 
 
-# Stand-alone measurement programs (register-only probes of the matrix pipe that the design notes
-# quote), built next to the objects: csrc/probes/NAME.hip -> csrc/build/NAME
-PROBES = ["mfma_ceiling"]
-
 # per-file additions; the prologue reproduces separately rounded fp32 products and sums
 EXTRA_FLAGS = {"qk_prologue.hip": ["-ffp-contract=off"]}
 
@@ -57,12 +53,6 @@ def build(verbose=True):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
-    for name in PROBES:
-        src = os.path.join(CSRC, "probes", name + ".hip")
-        if os.path.exists(src):
-            r = subprocess.run([_hipcc(), *FLAGS, src, "-o", os.path.join(OBJDIR, name)], capture_output=True, text=True)
-            if r.returncode != 0:
-                raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
     if verbose:
         print("built", LIB)
     return LIB

@@ -90,7 +90,7 @@ struct LaunchChoice {
   int policy;  // AttnParams::split_policy: 1 plain launch, 2 balanced when the planner offers a plan
 };
 
-LaunchChoice choose_launch(const xdit_attn_args* a, bool plain = false) {
+LaunchChoice choose_launch(const xdit_attn_args* a, bool plain = false, bool fold_only = false) {
   LaunchChoice best = {128, 1};
   const int D = kernel_head_dim(a->D);
   if (D == 0) return best;
@@ -124,16 +124,16 @@ LaunchChoice choose_launch(const xdit_attn_args* a, bool plain = false) {
       xdit::AttnParams q;
       std::memset(&q, 0, sizeof(q));
       q.Sk = (int)a->Sk; q.Sk2 = (int)a->Sk2; q.total_tiles = (int)tiles;
-      q.deterministic = a->deterministic;
+      q.streamed_ok = a->streamed_sharing != 0;
       q.split_policy = policy;
       if (policy == 2) {
-        xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8);
+        xdit::plan_split(q, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8, fold_only);
         if (q.split_units == 0) continue;  // no balanced plan for this shape
       } else if (a->balance == 2 && !plain) {
         // a balanced plan is to be taken when there is one: the plain launch only stands in without
         xdit::AttnParams t = q;
         t.split_policy = 2;
-        xdit::plan_split(t, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8);
+        xdit::plan_split(t, rows, slots, D, 2, fp8 ? 1 : xdit::kClaimsPerWorkgroup, !fp8, fold_only);
         if (t.split_units != 0) continue;
       }
       int64_t sharing = (tiles + cus - 1) / cus;  // workgroups on the busiest compute unit at once
@@ -146,12 +146,15 @@ LaunchChoice choose_launch(const xdit_attn_args* a, bool plain = false) {
       // partial results written and folded, in thousands of rows per compute unit
       const double parts = q.split_units ? (double)(tiles - q.split_full) * q.split_pmax * rows / cus * 1e-3 : 0.0;
       double cost;
+      // the ring step folds its shared tiles inside the attention kernel: a slice per workgroup at its end, or the whole
+      // tile by whoever completes it, one round trip to memory after the other (measured: about 25 us)
+      const double fold_us = fold_only && q.split_units ? 25.0 : 0.0;
       if (fp8) {
         const int cls = rows == 128 ? 5 - (int)sharing : i;
-        cost = kRateFp8[cls] * units * rows * (double)sharing * 1e-3 + kSegFp8[cls] * segs * (double)sharing + (q.split_units ? split_fp8_us + parts_fp8_us * parts : 0.0);
+        cost = kRateFp8[cls] * units * rows * (double)sharing * 1e-3 + kSegFp8[cls] * segs * (double)sharing + (q.split_units ? split_fp8_us + parts_fp8_us * parts : 0.0) + fold_us;
       } else {
         const int cls = rows == 128 ? (sharing > 1 ? 2 : 3) : i;
-        cost = rate[cls] * units * rows * (double)sharing * 1e-3 + seg_us[cls] * segs * (double)sharing + (q.split_units ? split_us + parts_us * parts : 0.0);
+        cost = rate[cls] * units * rows * (double)sharing * 1e-3 + seg_us[cls] * segs * (double)sharing + (q.split_units ? split_us + parts_us * parts : 0.0) + fold_us;
       }
       if (best_cost < 0 || cost < best_cost) { best.rows = rows; best.policy = policy; best_cost = cost; }
     }
@@ -300,34 +303,47 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.scale = a->softmax_scale;
   p.cu_count = a->cu_count;
-  p.deterministic = a->deterministic;
-  if (acc != nullptr) {  // folded in the epilogue of whole query tiles: no shared last round
+  p.streamed_ok = a->streamed_sharing != 0;
+  if (acc != nullptr) {
     p.acc_out = acc->acc_out; p.acc_lse = acc->acc_lse;
     p.ao_b = acc->acc_out_stride.b; p.ao_h = acc->acc_out_stride.h; p.ao_s = acc->acc_out_stride.s;
     p.al_b = acc->acc_lse_stride.b; p.al_h = acc->acc_lse_stride.h; p.al_s = acc->acc_lse_stride.s;
     p.acc_first = acc->first != 0;
     p.acc_store = acc->discard_acc_out == 0;
-  } else if (a->workspace != nullptr && a->workspace_bytes > 0 && aligned16(a->workspace)) {
+  }
+  if (a->workspace != nullptr && a->workspace_bytes >= (int64_t)xdit::kCounterRegionBytes && aligned16(a->workspace)) {
     p.ws_out = a->workspace;
     p.ws_preserved = a->workspace_preserved != 0;
     p.ws_bytes = (size_t)a->workspace_bytes;
   }
   hipStream_t stream = (hipStream_t)a->stream;
 
+  const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN;
+  if (fp8 && a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
+  if (!fp8 && !mfma16_path(a) && a->D > 128) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d above 128 is not implemented", a->D);
+  // A workspace whose contents the caller does not vouch for gets its counters cleared, whatever
+  // launch follows: the next call on it may then say "preserved" whether this one is balanced or not.
+  if (p.ws_out != nullptr && !p.ws_preserved) xdit::launch_counter_reset(p.ws_out, stream);
   hipError_t e;
-  if (mfma16_path(a)) {
-    p.d_actual = a->D;
-    const LaunchChoice c = choose_launch(a, acc != nullptr || p.ws_out == nullptr);  // no workspace: the shape that suits a plain launch
+  if (fp8 || mfma16_path(a)) {
+    const int D = fp8 ? 128 : kernel_head_dim(a->D);
+    if (!fp8) p.d_actual = a->D;
+    const bool fused = acc != nullptr;
+    LaunchChoice c = choose_launch(a, p.ws_out == nullptr, fused);  // no workspace: the shape that suits a plain launch
     p.split_policy = c.policy;
-    e = acc != nullptr ? xdit::launch_attn_fwd_16_ring(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), c.rows, stream)
-                       : xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, kernel_head_dim(a->D), c.rows, stream);
-  } else if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) {
-    if (a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
-    const LaunchChoice c = choose_launch(a, acc != nullptr || p.ws_out == nullptr);
-    p.split_policy = c.policy;
-    e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, c.rows, stream);
+    if (c.policy == 2) {
+      // a workspace too small for the chosen balanced plan: the best PLAIN launch, not that shape run plain
+      xdit::AttnParams plan;
+      const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, c.rows, &plan, fused) : xdit::attn_fwd_16_workspace(p, D, c.rows, &plan, fused);
+      if (need > p.ws_bytes) {
+        c = choose_launch(a, true, fused);
+        p.split_policy = c.policy;
+      }
+    }
+    if (fp8) e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, c.rows, stream);
+    else e = fused ? xdit::launch_attn_fwd_16_ring(p, a->dtype == XDIT_DTYPE_FP16, D, c.rows, stream)
+                   : xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, D, c.rows, stream);
   } else {
-    if (a->D > 128) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d above 128 is not implemented", a->D);
     e = xdit::launch_attn_fwd_f32(p, a->D, stream);  // fp32 tensors: every 16-bit case went to the 16-bit kernel
   }
   if (e != hipSuccess) return fail(XDIT_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
@@ -362,7 +378,13 @@ int xdit_attn_fwd_noalloc(const xdit_attn_args* a) {
     }
     b.workspace = ptr;
     b.workspace_bytes = (int64_t)XDIT_ATTN_NOALLOC_SCRATCH_BYTES;
-    b.workspace_preserved = 1;  // the array starts out zeroed and only this library writes it
+    // The array starts out zeroed and only this library writes it, so its counters are as the last
+    // call left them: at zero, unless that call failed part-way (then a kernel clears them first).
+    static std::atomic<int> scratch_dirty[xdit::kMaxDevices];
+    b.workspace_preserved = scratch_dirty[slot].load(std::memory_order_relaxed) == 0;
+    const int rc = attn_fwd_impl(&b, nullptr);
+    scratch_dirty[slot].store(rc != XDIT_OK, std::memory_order_relaxed);
+    return rc;
   }
   return attn_fwd_impl(&b, nullptr);
 }
@@ -389,7 +411,7 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.cu_count = a->cu_count;
-  p.deterministic = a->deterministic;
+  p.streamed_ok = a->streamed_sharing != 0;
   if (!(a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128) && !mfma16_path(a)) return 0;
   const LaunchChoice c = choose_launch(a);
   p.split_policy = c.policy;
@@ -415,7 +437,7 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
   std::memset(&p, 0, sizeof(p));
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.cu_count = a->cu_count;
-  p.deterministic = a->deterministic;
+  p.streamed_ok = a->streamed_sharing != 0;
   if (a->dtype == XDIT_DTYPE_FP32 && a->D > 0 && a->D % 8 == 0 && a->D <= 128) {
     // the fp32 kernel: one workgroup per query tile, no shared last round, no workspace
     const int rows = xdit::attn_fwd_f32_rows(p);
@@ -431,13 +453,15 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
     return XDIT_OK;
   }
   if (!fp8 && !b16) return fail(XDIT_ERR_UNSUPPORTED, "no launch plan for this dtype / head_dim");
-  const LaunchChoice choice = choose_launch(a);
+  const bool ring_step = out->ring_step != 0;
+  const LaunchChoice choice = choose_launch(a, false, ring_step);
   const int rows = choice.rows;
   p.split_policy = choice.policy;
-  const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q);
+  const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q, ring_step) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q, ring_step);
   const uint32_t size = out->struct_size;
   std::memset(out, 0, sizeof(*out));
   out->struct_size = size;
+  out->ring_step = ring_step;
   out->rows_per_workgroup = rows;
   out->query_tiles = q.total_tiles;
   out->kv_iterations = (int32_t)((a->Sk + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile + (a->Sk2 + xdit::kKeysPerTile - 1) / xdit::kKeysPerTile);
@@ -450,6 +474,8 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
   out->first_claimer = q.split_units ? (q.split_fuse0 <= q.split_full ? q.split_fuse0 : q.split_full) : 0;
   out->counter = xdit::split_counters(q) > 0 ? 1 : 0;
   out->streamed = q.split_dyn;
+  out->fold_in_kernel = q.split_fold;
+  out->parts_first = q.split_order;
   if (q.split_dyn) out->range_len = q.split_s0;
   out->workgroups = (int32_t)xdit::split_grid(q);
   return XDIT_OK;

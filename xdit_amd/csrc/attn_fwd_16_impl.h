@@ -91,6 +91,7 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
   const int nt1 = (pp->Sk + kKeysPerTile - 1) / kKeysPerTile;
   const int nt = nt1 + (pp->Sk2 + kKeysPerTile - 1) / kKeysPerTile;
   __shared__ unsigned ticket;   // range claims
+  __shared__ unsigned fold_post;  // fold duties: the slices this workgroup folds, posted by thread 0
   __shared__ int drawn[2];      // streamed sharing: KV tile of the stream position after next, by parity
   WorkgroupWalk walk;
   Segment seg;
@@ -220,7 +221,6 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
   };
   XDIT_TRACE_POINT(seg.slot >= 0, 0);
   open_segment(seg);
-
   for (;;) {  // segments of this workgroup
     // Coordinates of the segment being computed (open_segment of the next one overwrites them).
     const int cb = b, ch = h, cqt = qt;
@@ -418,7 +418,7 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
     const float lse = (m_used * c + fast_log2(l_tot)) * kLn2;
     XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + G::BUF_BYTES + wave * kStageBytes;
     const int row0 = cqt * kRowsPerBlock + wave * kRowsPerWave;   // first query row of this wavefront
-    if constexpr (!FUSED) {
+    if (!FUSED || part_out != nullptr) {
       // The normalised rows go out through LDS, 64 columns at a time: lane (query, half) writes
       // its 4-element pieces into a [32 rows][64 columns] block private to the wavefront, which is
       // read back with 8 lanes per row, so that every global store covers whole 128-byte lines of
@@ -463,13 +463,16 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
           const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
           // streaming stores: the rows are not read again by this kernel, and lines that leave the
           // cache as they are written are not left for the write-back at the kernel's end
-          if (row < rows_live && col < cols_live) __builtin_nontemporal_store(x, (vec8*)(obase + row * ostride + col));
+          if (row < rows_live && col < cols_live) {
+            if (FUSED && part_out != nullptr) store16_device(obase + row * ostride + col, __builtin_bit_cast(i32x4, x));  // read by another workgroup of this launch
+            else __builtin_nontemporal_store(x, (vec8*)(obase + row * ostride + col));
+          }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         __builtin_amdgcn_wave_barrier();
       }
       if (hh == 0 && cqrow < pp->Sq) {
-        if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
+        if (part_out != nullptr) { if (FUSED) store_float_device(part_lse + wave * kRowsPerWave + l32, lse); else part_lse[wave * kRowsPerWave + l32] = lse; }
         else if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = lse;
       }
     } else {
@@ -544,13 +547,31 @@ __device__ __forceinline__ void attn_workgroup(unsigned char* smem) {
       }
     }
     XDIT_TRACE_POINT(seg.slot >= 0, 3);
+    if constexpr (FUSED && NW != 12) if (seg.slot >= 0 && pp->split_fold != 0) {
+      // this part of a shared tile is written: its arrival, with its fold duty unless that waits for the workgroup's end
+      const WalkGeom g = walk_geom(pp);
+      const int r = seg.tile - g.split_full;
+      const int j = (int)(seg.slot - (int64_t)r * g.split_pmax);
+      const int n = shared_tile_parts(g, nt, r);
+      const bool now = g.split_order == 0;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's rows of the partial result have been written through
+      fold_arrival<T, D, kRowsPerBlock, FUSED>(pp, nt, r, j, n, now, &fold_post);
+    }
     if (!more) break;
-    if (PAD) {  // the staging blocks lay over the second K/V buffer: clear it again (the barrier of the first iteration orders this)
+    if (PAD) {
+      // The staging blocks lay over the second K/V buffer: clear it again.  The clearing is striped over the whole
+      // buffer, so every wavefront must be done with its staging block first; the barrier of the next segment's first
+      // iteration orders the clearing against that segment's tile loads.
+      __syncthreads();
       typedef __attribute__((ext_vector_type(4))) int i32x4;
       const i32x4 zero = {0, 0, 0, 0};
       for (int i = (wave * 64 + lane) * 16; i < G::BUF_BYTES; i += 64 * kWaves * 16) *(XDIT_LDS i32x4*)((XDIT_LDS unsigned char*)smem + G::BUF_BYTES + i) = zero;
     }
     seg = next_seg;
+  }
+  if constexpr (FUSED && NW != 12) if (pp->split_fold != 0) {
+    if (pp->split_order != 0) fold_duties_at_end<T, D, kRowsPerBlock, FUSED>(pp, nt, &fold_post);
+    if (walk.claimer && pp->split_counter != nullptr && pp->split_dyn == 0) claimer_done(pp);
   }
 }
 
@@ -585,11 +606,8 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  // the ring step folds in the epilogue of whole query tiles: no shared last round
-  bind_workspace(q, p, FUSED ? 0 : plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, kClaimsPerWorkgroup, true), rows, D, 2);
-  if constexpr (!FUSED) {
-    launch_counter_reset(q, stream);
-  }
+  // the ring step takes a balanced plan only when the attention kernel folds the parts itself (the fold goes on into the accumulator)
+  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, kClaimsPerWorkgroup, true, FUSED), rows, D, 2);
   if (q.d_actual == D) q.d_actual = 0;
   // computed head_dims built for tensors smaller than D: 80, 96, 112 (and 128) of 128; 32 (and 64) of 64
   hipError_t e;
@@ -605,7 +623,7 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   }
   if (e != hipSuccess) return e;
   if constexpr (!FUSED) {
-    if (q.split_units) {
+    if (q.split_units && !q.split_fold) {  // tiles of many parts: folded by a launch of its own
       const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
       const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
       hipLaunchKernelGGL((attn_combine_kernel<T, D>), cgrid, dim3(256), 0, stream, q, rows, nt, split_counters(q));

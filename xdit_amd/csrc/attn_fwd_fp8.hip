@@ -59,7 +59,8 @@ constexpr int lds_bytes() { return BUF_BYTES + (BUF_BYTES > NW * kStageBytes ? B
 // whole 128-byte lines.
 // FUSED: the ring step; the block (rounded to TO, what a block_out tensor would have held) is
 // folded into the fp32 accumulator with the arithmetic of the merge kernel, so that the result
-// equals forward + merge bit for bit; such a launch has whole query tiles only.
+// equals forward + merge bit for bit; the parts of shared tiles go through the workspace as in a plain
+// forward and are folded, then folded into the accumulator, by the fold duties.
 template <typename TO, int NW, bool FUSED>
 __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
   typedef unsigned char u8;
@@ -70,6 +71,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
   const int nt1 = (pp->Sk + kKeysPerTile - 1) / kKeysPerTile;
   const int nt = nt1 + (pp->Sk2 + kKeysPerTile - 1) / kKeysPerTile;
   __shared__ unsigned ticket;
+  __shared__ unsigned fold_post;  // fold duties: the slices this workgroup folds, posted by thread 0
   WorkgroupWalk walk;
   Segment seg;
   {
@@ -174,7 +176,6 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
     issue_tile(sg.it0, 0);
   };
   open_segment(seg);
-
   for (;;) {  // segments of this workgroup
     const int cb = b, ch = h, cqt = qt;
     const float cc = c, csv = sv;
@@ -349,7 +350,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
     typedef __attribute__((ext_vector_type(8))) TO vec8;
     XDIT_LDS unsigned char* stage = (XDIT_LDS unsigned char*)smem + BUF_BYTES + wave * kStageBytes;
     const int row0 = cqt * kRowsPerBlock + wave * kRowsPerWave;
-    if constexpr (!FUSED) {
+    if (!FUSED || part_out != nullptr) {
       TO* obase;
       int64_t ostride;
       int rows_live = kRowsPerWave;
@@ -381,13 +382,16 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
         for (int r = 0; r < 4; r++) {
           const int row = rd_row + 8 * r;
           const vec8 x = *(const XDIT_LDS vec8*)(stage + row * kStagePitch + rd_col * 2);
-          if (row < rows_live) __builtin_nontemporal_store(x, (vec8*)(obase + row * ostride + 64 * half + rd_col));
+          if (row < rows_live) {
+            if (FUSED && part_out != nullptr) store16_device(obase + row * ostride + 64 * half + rd_col, __builtin_bit_cast(i32x4, x));  // read by another workgroup of this launch
+            else __builtin_nontemporal_store(x, (vec8*)(obase + row * ostride + 64 * half + rd_col));
+          }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         __builtin_amdgcn_wave_barrier();
       }
       if (hh == 0 && cqrow < pp->Sq) {
-        if (part_out != nullptr) part_lse[wave * kRowsPerWave + l32] = lse;
+        if (part_out != nullptr) { if (FUSED) store_float_device(part_lse + wave * kRowsPerWave + l32, lse); else part_lse[wave * kRowsPerWave + l32] = lse; }
         else if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = lse;
       }
     } else {
@@ -455,8 +459,22 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
         if (pp->lse != nullptr) pp->lse[cb * pp->ls_b + ch * pp->ls_h + cqrow] = new_lse;
       }
     }
+    if constexpr (FUSED && NW != 12) if (seg.slot >= 0 && pp->split_fold != 0) {
+      // this part of a shared tile is written: its arrival, with its fold duty unless that waits for the workgroup's end
+      const WalkGeom g = walk_geom(pp);
+      const int r = seg.tile - g.split_full;
+      const int j = (int)(seg.slot - (int64_t)r * g.split_pmax);
+      const int n = shared_tile_parts(g, nt, r);
+      const bool now = g.split_order == 0;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's rows of the partial result have been written through
+      fold_arrival<TO, D, kRowsPerBlock, FUSED>(pp, nt, r, j, n, now, &fold_post);
+    }
     if (!more) break;
     seg = next_seg;
+  }
+  if constexpr (FUSED && NW != 12) if (pp->split_fold != 0) {
+    if (pp->split_order != 0) fold_duties_at_end<TO, D, kRowsPerBlock, FUSED>(pp, nt, &fold_post);
+    if (walk.claimer && pp->split_counter != nullptr && pp->split_dyn == 0) claimer_done(pp);
   }
 }
 
@@ -476,9 +494,8 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  // the ring step folds in the epilogue of whole query tiles: no shared last round
-  bind_workspace(q, p, FUSED ? 0 : plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1), rows, D, 2);
-  if constexpr (!FUSED) launch_counter_reset(q, stream);
+  // the ring step takes a balanced plan only when the attention kernel folds the parts itself (the fold goes on into the accumulator)
+  bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1, false, FUSED), rows, D, 2);
   static std::atomic<bool> lds_ready[kMaxDevices];
   constexpr int lds = lds_bytes<NW>();
   const int slot = current_device_slot();
@@ -490,7 +507,7 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   dim3 grid(split_grid(q));
   hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW, FUSED>), grid, dim3(64 * NW), lds, stream, q);
   if constexpr (!FUSED) {
-    if (q.split_units) {
+    if (q.split_units && !q.split_fold) {  // tiles of many parts: folded by a launch of its own
       const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
       const dim3 cgrid((unsigned)((rows * (D / 8) + 255) / 256), (unsigned)(q.total_tiles - q.split_full));
       hipLaunchKernelGGL((attn_combine_kernel<TO, D>), cgrid, dim3(256), 0, stream, q, rows, nt, split_counters(q));
@@ -500,13 +517,13 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
 }
 
 template <int NW>
-static size_t workspace_one(const AttnParams& p, AttnParams* plan) {
+static size_t workspace_one(const AttnParams& p, AttnParams* plan, bool fold_only) {
   AttnParams q = p;
   constexpr int rows = kRowsPerWave * NW;
   q.nq_tiles = (p.Sq + rows - 1) / rows;
   q.total_tiles = p.B * p.H * q.nq_tiles;
   q.tiles_per_xcd = (q.total_tiles + 7) / 8;
-  const size_t need = plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1);
+  const size_t need = plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1, false, fold_only);
   if (plan != nullptr) *plan = q;
   return need;
 }
@@ -527,11 +544,11 @@ hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_pe
   return p.acc_out != nullptr ? launch_fp8<true>(p, out_is_fp16, rows_per_block, stream) : launch_fp8<false>(p, out_is_fp16, rows_per_block, stream);
 }
 
-size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan) {
+size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan, bool fold_only) {
   using namespace fp8path;
-  if (rows_per_block == 384) return workspace_one<12>(p, plan);
-  if (rows_per_block == 256) return workspace_one<8>(p, plan);
-  return workspace_one<4>(p, plan);
+  if (rows_per_block == 384) return workspace_one<12>(p, plan, fold_only);
+  if (rows_per_block == 256) return workspace_one<8>(p, plan, fold_only);
+  return workspace_one<4>(p, plan, fold_only);
 }
 
 }  // namespace xdit

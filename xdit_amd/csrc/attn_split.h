@@ -1,7 +1,8 @@
 // Balanced launch shared by the attention kernels: when the query tiles do not fill a whole
 // number of rounds of resident workgroups, the KV iterations of the last round's tiles are cut
 // into equal ranges, one per workgroup; partial (out, lse) pairs go through a workspace and are
-// folded by attn_combine_kernel.
+// folded by the workgroups of the attention kernel themselves (fold duties) or, for tiles of many
+// parts, by attn_combine_kernel.
 #pragma once
 #include <atomic>
 
@@ -28,45 +29,13 @@ __device__ __forceinline__ unsigned draw_ticket(unsigned* counter) {
 
 // The launch geometry the walker reads, gathered from the kernel arguments when needed.
 struct WalkGeom {
-  int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers, split_dyn, split_s0;
+  int total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax, split_fuse0, split_claimers, split_dyn, split_s0, split_order;
 };
 typedef const __attribute__((address_space(4))) AttnParams* ParamsPtr;
 __device__ __forceinline__ WalkGeom walk_geom(ParamsPtr pp) {
   WalkGeom g = {pp->total_tiles, pp->tiles_per_xcd, pp->split_full, pp->split_units, pp->split_len, pp->split_pmax,
-                pp->split_fuse0, pp->split_claimers, pp->split_dyn, pp->split_s0};
+                pp->split_fuse0, pp->split_claimers, pp->split_dyn, pp->split_s0, pp->split_order};
   return g;
-}
-
-// Runs the segments of this workgroup (see WorkgroupWalk in attn_walk.h for who does what).
-// `seg(tile, it0, it1, part_out, part_lse)` processes KV tiles [it0, it1) of query tile `tile`;
-// part_out == nullptr means "write the final result", otherwise the normalised partial result and
-// its log-sum-exp go to that workspace slot.  TO is the output element type, ROWS the query rows
-// per workgroup.
-template <typename TO, int ROWS, int D, typename Seg>
-__device__ __forceinline__ void run_workgroup(const AttnParams& p, Seg seg) {
-  const int nt = (p.Sk + kKeysPerTile - 1) / kKeysPerTile + (p.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
-  __shared__ unsigned ticket;
-  WorkgroupWalk walk;
-  if (!walk.start(p, nt, (int)blockIdx.x)) return;
-  bool first = true;
-  Segment s;
-  while (walk.next(p, nt, s)) {  // one segment per turn; a single call site keeps one copy of the kernel body
-    TO* part_out = nullptr;
-    float* part_lse = nullptr;
-    if (s.slot >= 0) {
-      part_out = (TO*)p.ws_out + s.slot * ROWS * D;
-      part_lse = p.ws_lse + s.slot * ROWS;
-    }
-    if (!first) __syncthreads();  // every wavefront is done with the LDS buffers of the previous segment
-    seg(s.tile, s.it0, s.it1, part_out, part_lse);
-    first = false;
-    if (walk.wants_claim(p.split_counter != nullptr)) {
-      __syncthreads();  // everyone has read the ticket of the previous claim
-      if (threadIdx.x == 0) ticket = atomicAdd(p.split_counter, 1u);
-      __syncthreads();
-      walk.claimed(p, ticket);
-    }
-  }
 }
 
 // Clears the counters of a balanced launch (a kernel, not a memset, so that the sequence can be
@@ -75,8 +44,90 @@ static __global__ void attn_counter_reset_kernel(unsigned* counter, int n) {
   for (int i = threadIdx.x; i < n; i += blockDim.x) counter[i] = 0u;
 }
 
-// Folds the parts of every query tile that was split: out = sum_k exp(lse_k - L) out_k,
-// L = log sum_k exp(lse_k), in fp32; one thread per 8 head_dim elements of a row.
+// Partial results that are folded inside the same launch cross from one XCD to another, whose L2
+// caches are not coherent with each other for ordinary accesses.  They are therefore written and
+// read with device-scope (relaxed atomic) accesses of 8 bytes, which the L2 passes through to
+// memory, instead of ordinary accesses bracketed by device-scope fences: such a fence writes back
+// (release) or invalidates (acquire) the whole L2 of the XCD, which cost the Flux step 30-45 us.
+// Order is kept by hand: a wavefront waits for its stores to complete (s_waitcnt vmcnt(0)) before
+// the workgroup barrier that precedes the arrival's atomic add, and the loads are issued after the
+// barrier that follows it.
+__device__ __forceinline__ void store16_device(void* p, i32x4 x) {
+  unsigned long long lo = ((unsigned long long)(unsigned)x[1] << 32) | (unsigned)x[0];
+  unsigned long long hi = ((unsigned long long)(unsigned)x[3] << 32) | (unsigned)x[2];
+  __hip_atomic_store((unsigned long long*)p, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((unsigned long long*)p + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ i32x4 load16_device(const void* p) {
+  const unsigned long long lo = __hip_atomic_load((const unsigned long long*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long hi = __hip_atomic_load((const unsigned long long*)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  i32x4 x = {(int)(unsigned)lo, (int)(unsigned)(lo >> 32), (int)(unsigned)hi, (int)(unsigned)(hi >> 32)};
+  return x;
+}
+__device__ __forceinline__ void store_float_device(float* p, float x) { __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float load_float_device(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// One (row, 8-column chunk) of a shared query tile folded from its parts:
+//   out = sum_k exp(lse_k - L) out_k / sum_k exp(lse_k - L),  lse = L + log sum_k exp(lse_k - L),  L = max_k lse_k,
+// in fp32, the parts taken in slot order.  `part0` / `lsep` point at this chunk / row in part 0;
+// parts are `out_stride` elements / `lse_stride` floats apart.  Eight parts are in flight per
+// thread (outputs and log-sum-exps loaded together, so a tile of up to eight parts costs one round
+// trip to memory); the running maximum L is carried from one group of eight to the next as in the
+// online softmax.  Used by attn_combine_kernel and by the fold inside the attention kernels, so
+// that both give the same bits.  DEVICE: the parts were written by other workgroups of this launch
+// (device-scope loads, see above).
+template <typename T, bool DEVICE>
+__device__ __forceinline__ void combine_item(const T* part0, const float* lsep, int nparts, int64_t out_stride, int64_t lse_stride,
+                                             __attribute__((ext_vector_type(8))) T& o, float& lse_out) {
+  typedef __attribute__((ext_vector_type(8))) T vec8;
+  float L = -INFINITY;
+  float denom = 0.f;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < nparts; k0 += 8) {
+    vec8 x[8];
+    float ls[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int k = k0 + j < nparts ? k0 + j : nparts - 1;
+      if constexpr (DEVICE) {
+        x[j] = __builtin_bit_cast(vec8, load16_device(part0 + (int64_t)k * out_stride));
+        ls[j] = load_float_device(lsep + (int64_t)k * lse_stride);
+      } else {
+        x[j] = *(const vec8*)(part0 + (int64_t)k * out_stride);
+        ls[j] = lsep[(int64_t)k * lse_stride];
+      }
+    }
+    float Ln = L;
+#pragma unroll
+    for (int j = 0; j < 8; j++) Ln = fmaxf(Ln, ls[j]);
+    const float keep = __expf(L - Ln);  // 0 on the first group (L = -inf)
+    L = Ln;
+    denom *= keep;
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] *= keep;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float w = k0 + j < nparts ? __expf(ls[j] - L) : 0.f;
+      denom += w;
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[i] += w * (float)x[j][i];
+    }
+  }
+  const float inv = 1.0f / denom;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    // the product is rounded to fp32 and THEN to T wherever this is inlined: left alone, the compiler
+    // takes a multiply that rounds straight to fp16 in some contexts and not in others (one unit in
+    // the last place apart in about one element of 10^4)
+    float t = acc[i] * inv;
+    asm volatile("" : "+v"(t));
+    o[i] = (T)t;
+  }
+  lse_out = L + __logf(denom);
+}
+
+// Folds the parts of every query tile that was split (launches whose tiles have more parts than
+// the attention kernel folds itself); one thread per 8 head_dim elements of a row.
 // grid = (ceil(rows_per_block * D/8 / 256), shared query tiles): blockIdx.y is the tile, so the
 // tile's coordinates and part range are wavefront-uniform.
 template <typename T, int D>
@@ -102,43 +153,151 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnParams p, c
   const float* lsep = p.ws_lse + ((int64_t)r * p.split_pmax) * rows_per_block + row;
   typedef __attribute__((ext_vector_type(8))) T vec8;
   const T* part0 = (const T*)p.ws_out + (((int64_t)r * p.split_pmax) * rows_per_block + row) * D + col;
-  // One pass, eight parts in flight per thread (outputs and log-sum-exps are loaded together,
-  // so a tile of up to eight parts costs one round trip to memory); the running maximum L is
-  // carried from one group of eight to the next as in the online softmax.
-  float L = -INFINITY;
-  float denom = 0.f;
-  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < nparts; k0 += 8) {
-    vec8 x[8];
-    float ls[8];
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const int k = k0 + j < nparts ? k0 + j : nparts - 1;
-      x[j] = *(const vec8*)(part0 + (int64_t)k * rows_per_block * D);
-      ls[j] = lsep[(int64_t)k * rows_per_block];
+  vec8 o;
+  float lse;
+  combine_item<T, false>(part0, lsep, nparts, (int64_t)rows_per_block * D, rows_per_block, o, lse);
+  *(vec8*)((T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s + col) = o;
+  if (col == 0 && p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = lse;
+}
+
+// ---- the fold inside the attention kernels (fold duties, see attn_walk.h) ----------------------
+// Counter region of a workspace (4096 words): [0, kArriveBase) the range counter of a launch or
+// the per-tile counters of streamed sharing; [kArriveBase, kDoneIndex) one fold word per shared
+// tile; kDoneIndex counts the claimers that have finished (its last one clears the range counter).
+constexpr int kArriveBase = 2048;
+constexpr int kDoneIndex = 4095;
+
+// Rows of shared tile r (the slices in `mask`, n parts) folded by all threads of the workgroup and
+// written to the output tensors, or, FUSED (the ring step), folded further into the fp32
+// accumulator with the arithmetic of the merge kernel on the folded block rounded to T.  The
+// D/8 chunks of a row are held by adjacent lanes of one wavefront in the same pass, so every lane
+// of a row has read the accumulated log-sum-exp before the row's first lane overwrites it.
+template <typename T, int D, int ROWS, bool FUSED>
+__device__ __forceinline__ void fold_tile_slices(ParamsPtr pp, int nt, int r, unsigned mask, int n) {
+  constexpr int TPR = D / 8;
+  typedef __attribute__((ext_vector_type(8))) T vec8;
+  const int tid = (int)threadIdx.x, nthreads = (int)blockDim.x;
+  const int nq_tiles = pp->nq_tiles, H = pp->H, Sq = pp->Sq, dact = pp->d_actual, pmax = pp->split_pmax;
+  const int tile = pp->split_full + r;
+  const int bh = tile / nq_tiles;
+  const int qt = tile - bh * nq_tiles;
+  const int b = bh / H;
+  const int h = bh - b * H;
+  const T* const parts = (const T*)pp->ws_out + ((int64_t)r * pmax) * ROWS * D;
+  const float* const lses = pp->ws_lse + ((int64_t)r * pmax) * ROWS;
+  const bool all = mask == (n >= 32 ? 0xffffffffu : (1u << n) - 1u);
+  for (int j = 0; j < n; j++) {
+    int r0 = 0, r1 = ROWS;
+    if (!all) {
+      if (!((mask >> j) & 1u)) continue;
+      fold_slice_rows(j, n, ROWS, r0, r1);
     }
-    float Ln = L;
+    for (int item = tid; item < (r1 - r0) * TPR; item += nthreads) {
+      const int row = r0 + item / TPR;
+      const int col = (item % TPR) * 8;
+      const int qrow = qt * ROWS + row;
+      if (qrow >= Sq || (dact != 0 && col >= dact)) continue;
+      vec8 o;
+      float lse;
+      combine_item<T, true>(parts + (int64_t)row * D + col, lses + row, n, (int64_t)ROWS * D, ROWS, o, lse);
+      if constexpr (!FUSED) {
+        *(vec8*)((T*)pp->out + b * pp->os_b + h * pp->os_h + (int64_t)qrow * pp->os_s + col) = o;
+        if (col == 0 && pp->lse != nullptr) pp->lse[b * pp->ls_b + h * pp->ls_h + qrow] = lse;
+      } else {
+        const bool first = pp->acc_first != 0;
+        float* alp = pp->acc_lse + b * pp->al_b + h * pp->al_h + (int64_t)qrow * pp->al_s;
+        float* aptr = pp->acc_out + b * pp->ao_b + h * pp->ao_h + (int64_t)qrow * pp->ao_s + col;
+        f32x4 m0, m1;
 #pragma unroll
-    for (int j = 0; j < 8; j++) Ln = fmaxf(Ln, ls[j]);
-    const float keep = __expf(L - Ln);  // 0 on the first group (L = -inf)
-    L = Ln;
-    denom *= keep;
+        for (int e = 0; e < 4; e++) { m0[e] = (float)o[e]; m1[e] = (float)o[4 + e]; }
+        float new_lse = lse;
+        if (!first) {
+          const float la = *alp;  // read by every lane of the row before its first lane stores below
+          const float w = sigmoid(lse - la);
+          new_lse = la - log_sigmoid(la - lse);
+          const f32x4 a0 = *(const f32x4*)aptr, a1 = *(const f32x4*)(aptr + 4);
 #pragma unroll
-    for (int i = 0; i < 8; i++) acc[i] *= keep;
+          for (int e = 0; e < 4; e++) { m0[e] = fold_value(a0[e], m0[e], w); m1[e] = fold_value(a1[e], m1[e], w); }
+        }
+        if (pp->acc_store) { *(f32x4*)aptr = m0; *(f32x4*)(aptr + 4) = m1; }
+        if (pp->out != nullptr) {
+          vec8 y;
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const float w = k0 + j < nparts ? __expf(ls[j] - L) : 0.f;
-      denom += w;
-#pragma unroll
-      for (int i = 0; i < 8; i++) acc[i] += w * (float)x[j][i];
+          for (int e = 0; e < 4; e++) { y[e] = (T)m0[e]; y[4 + e] = (T)m1[e]; }
+          *(vec8*)((T*)pp->out + b * pp->os_b + h * pp->os_h + (int64_t)qrow * pp->os_s + col) = y;
+        }
+        if (col == 0) {
+          *alp = new_lse;
+          if (pp->lse != nullptr) pp->lse[b * pp->ls_b + h * pp->ls_h + qrow] = new_lse;
+        }
+      }
+    }
+    if (all) break;
+  }
+}
+
+// One event on the fold word of shared tile r by this workgroup (every thread calls it):
+// `arrival`: part j of the tile's n parts has just been written by this workgroup (with_duty: its
+// fold duty is presented with it); otherwise the duty of part j is presented on its own.  Folds
+// what the protocol hands this workgroup.  `post` is one word of LDS.
+template <typename T, int D, int ROWS, bool FUSED>
+__device__ __forceinline__ void fold_event_body(ParamsPtr pp, int nt, int r, int j, int n, bool arrival, bool with_duty, unsigned* post) {
+  __syncthreads();  // every wavefront's rows of the partial result have been stored (and awaited by it); `post` is free
+  if (threadIdx.x == 0) {
+    unsigned* const word = pp->ws_counters + kArriveBase + r;
+    const unsigned add = arrival ? fold_arrive_word(j, with_duty) : fold_duty_word(j);
+    const unsigned old = __hip_atomic_fetch_add(word, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (fold_last_event(old, add, n)) {  // nobody touches the tile's counters after this event
+      __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (pp->split_dyn) __hip_atomic_store(pp->ws_counters + r, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    *post = arrival ? fold_after_arrival(old, j, with_duty, n) : fold_after_duty(old, j, n);
+  }
+  __syncthreads();
+  const unsigned mask = (unsigned)__builtin_amdgcn_readfirstlane((int)*post);
+  if (mask != 0u) {
+    fold_tile_slices<T, D, ROWS, FUSED>(pp, nt, r, mask, n);
+  }
+}
+
+// The arrival of part j of shared tile r, called by the attention kernels after the part's rows are
+// stored.
+template <typename T, int D, int ROWS, bool FUSED>
+__device__ __forceinline__ void fold_arrival(ParamsPtr pp, int nt, int r, int j, int n, bool with_duty, unsigned* post) {
+  fold_event_body<T, D, ROWS, FUSED>(pp, nt, r, j, n, true, with_duty, post);
+}
+
+// At the very end of a workgroup of a parts-first launch: the fold duties of the parts it wrote at
+// its start.  Claimer c = workgroup split_fuse0 + c of such a launch has range c, whose (up to
+// two) parts are worked out again here rather than carried through the KV loops.
+template <typename T, int D, int ROWS, bool FUSED>
+__device__ __forceinline__ void fold_duties_at_end(ParamsPtr pp, int nt, unsigned* post) {
+  const WalkGeom g = walk_geom(pp);
+  const int u = (int)blockIdx.x - g.split_fuse0;
+  if (u < 0 || u >= g.split_units) return;
+  const int rem_iters = (g.total_tiles - g.split_full) * nt;
+  int lin = u * g.split_len;
+  const int lin_end = lin + g.split_len < rem_iters ? lin + g.split_len : rem_iters;
+  while (lin < lin_end) {
+    const int r = lin / nt;
+    const int it1 = lin_end - r * nt < nt ? lin_end - r * nt : nt;
+    const int j = u - (r * nt) / g.split_len;
+    fold_event_body<T, D, ROWS, FUSED>(pp, nt, r, j, shared_tile_parts(g, nt, r), false, false, post);
+    lin = r * nt + it1;
+  }
+}
+
+// At the very end of a claimer of a launch that hands ranges out through a counter and folds in
+// the kernel: the last claimer to finish puts the range counter (and this count) back to zero.
+__device__ __forceinline__ void claimer_done(ParamsPtr pp) {
+  if (threadIdx.x == 0) {
+    unsigned* const done = pp->ws_counters + kDoneIndex;
+    const unsigned old = __hip_atomic_fetch_add(done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((int)old == pp->split_claimers - 1) {
+      __hip_atomic_store(done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(pp->ws_counters, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-  const float inv = 1.0f / denom;
-  vec8 o;
-#pragma unroll
-  for (int i = 0; i < 8; i++) o[i] = (T)(acc[i] * inv);
-  *(vec8*)((T*)p.out + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_s + col) = o;
-  if (col == 0 && p.lse != nullptr) p.lse[b * p.ls_b + h * p.ls_h + qrow] = L + __logf(denom);
 }
 
 // State cached per device (a process may drive several): index of the current device.
@@ -198,16 +357,33 @@ static inline size_t split_parts_bytes(const AttnParams& q, int rows, int D, int
   return (size_t)(q.total_tiles - q.split_full) * q.split_pmax * rows * ((size_t)D * out_bytes + 4);
 }
 
-static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int out_bytes, int claims, bool streamed = false) {
+// The ring step folds the parts of its shared tiles inside the attention kernel (fold duties,
+// attn_walk.h: its fold goes on into the accumulator), which takes tiles of few parts; a plain
+// forward leaves them to attn_combine_kernel, a launch of its own (measured on Flux-1024 and on
+// three of its heads the fold inside the kernel was 6-8 % slower: whoever folds a tile reads all
+// of its parts alone, one round trip to memory after the other, at the very end of the launch).
+// Also whether the claimers take their range before their whole tile (possible when every claimer
+// has exactly one range and a whole tile; the parts are then complete long before the workgroups
+// end, and each folds its slice there instead of the last one folding everything).
+static inline void plan_fold(AttnParams& q) {
+  const int rem = q.total_tiles - q.split_full;
+  q.split_fold = q.split_units != 0 && q.split_pmax <= kFoldMaxParts && rem < kDoneIndex - kArriveBase ? 1 : 0;
+  q.split_order = q.split_fold && !q.split_dyn && q.split_units <= q.split_claimers && q.split_fuse0 <= q.split_full ? 1 : 0;
+}
+
+// `fold_only`: offer a plan only if the attention kernel folds the parts itself (the ring step,
+// whose fold goes on into the accumulator).
+static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int out_bytes, int claims, bool streamed = false, bool fold_only = false) {
   q.split_units = q.split_full = q.split_len = q.split_pmax = q.split_share = q.split_claimers = 0;
   q.split_fuse0 = 0x7fffffff;
   q.split_counter = nullptr;
-  q.split_dyn = q.split_s0 = 0;
+  q.split_dyn = q.split_s0 = q.split_order = q.split_fold = 0;
   const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
   const int T = q.total_tiles;
   const int full = (T / slots) * slots;
   const int rem = T - full;
   if (rem == 0 || nt < 8) return 0;
+  if (fold_only && rows > 256) return 0;  // the 12-wavefront ring-step kernels have no registers to spare for the fold
   int share = (int)(((int64_t)rem * nt + slots - 1) / slots);  // iterations per workgroup
   if (share < 4) share = 4;
   // Iterations of the critical path saved by filling the last round: a plan is offered when it
@@ -216,9 +392,9 @@ static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int o
   if (q.split_policy == 1 || nt - share < kMinSaving) return 0;
   // Few shared tiles with short shares: streamed sharing.  Every resident workgroup joins the
   // group of one shared tile; unless the caller asks for bit-reproducible results.
-  if (streamed && !q.deterministic && share < 2 * kMinClaimLen && rem * 4 <= slots) {
+  if (streamed && q.streamed_ok && share < 2 * kMinClaimLen && rem * 4 <= slots) {
     const int pmax = (slots + rem - 1) / rem;
-    if (pmax * kStreamedOwn * 2 <= nt && (size_t)rem * 4 <= kCounterRegionBytes) {
+    if (pmax * kStreamedOwn * 2 <= nt && rem <= kArriveBase && (!fold_only || pmax <= kFoldMaxParts)) {
       q.split_full = full;
       q.split_units = q.split_claimers = slots;
       q.split_len = share;
@@ -227,6 +403,7 @@ static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int o
       q.split_fuse0 = full >= slots ? full - slots : 0x7fffffff;
       q.split_dyn = 1;
       q.split_s0 = kStreamedOwn;
+      if (fold_only) plan_fold(q);
       return kCounterRegionBytes + split_parts_bytes(q, rows, D, out_bytes);
     }
   }
@@ -248,6 +425,12 @@ static inline size_t plan_split(AttnParams& q, int rows, int slots, int D, int o
   q.split_pmax = (nt + len - 1) / len + 1;
   q.split_claimers = claimers;
   q.split_fuse0 = full >= claimers ? full - claimers : 0x7fffffff;
+  if (fold_only) plan_fold(q);
+  if (fold_only && !q.split_fold) {
+    q.split_units = q.split_full = q.split_len = q.split_pmax = q.split_share = q.split_claimers = 0;
+    q.split_fuse0 = 0x7fffffff;
+    return 0;
+  }
   return kCounterRegionBytes + split_parts_bytes(q, rows, D, out_bytes);
 }
 
@@ -258,7 +441,7 @@ static inline void bind_workspace(AttnParams& q, const AttnParams& p, size_t nee
     q.split_units = q.split_full = q.split_len = q.split_pmax = q.split_share = q.split_claimers = 0;
     q.split_fuse0 = 0x7fffffff;
     q.split_counter = nullptr;
-    q.split_dyn = q.split_s0 = 0;
+    q.split_dyn = q.split_s0 = q.split_order = q.split_fold = 0;
     q.ws_out = nullptr;
   } else {
     const size_t rem = (size_t)(q.total_tiles - q.split_full);
@@ -269,13 +452,11 @@ static inline void bind_workspace(AttnParams& q, const AttnParams& p, size_t nee
   }
 }
 
-// The launches around the attention kernel of a balanced launch.  Counters must be zero when the
-// attention kernel starts: a workspace whose contents the caller vouches for (ws_preserved: left
-// as this library's previous call on it left them) has them at zero already, since the fold
-// kernel clears what its launch used; otherwise a small kernel clears the whole region first.
-static inline void launch_counter_reset(const AttnParams& q, hipStream_t stream) {
-  if (q.split_units != 0 && !q.ws_preserved)
-    hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(256), 0, stream, q.ws_counters, (int)(kCounterRegionBytes / 4));
+// Clears the counter region of a workspace whose contents the caller does not vouch for.  Done by
+// the C entry points for EVERY call that is given such a workspace, balanced or not, so that
+// "preserved" means the same whatever the earlier calls on the workspace were.
+static inline void launch_counter_reset(void* workspace, hipStream_t stream) {
+  hipLaunchKernelGGL(attn_counter_reset_kernel, dim3(1), dim3(256), 0, stream, (unsigned*)workspace, (int)(kCounterRegionBytes / 4));
 }
 
 // Workgroups of a launch planned by plan_split (after bind_workspace).

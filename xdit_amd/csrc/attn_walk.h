@@ -36,7 +36,7 @@ struct Segment {
 
 // The sequence of segments of workgroup `w`.  P is any struct with the launch-geometry members of
 // AttnParams (total_tiles, tiles_per_xcd, split_full, split_units, split_len, split_pmax,
-// split_fuse0, split_claimers, split_dyn, split_s0); `nt` is the number of KV iterations of a
+// split_fuse0, split_claimers, split_dyn, split_s0, split_order); `nt` is the number of KV iterations of a
 // whole tile.
 // Plain launch (split_units == 0): workgroup = one query tile over all KV iterations.  Balanced
 // launch: the first split_full workgroups each take a whole query tile; the KV iterations of the
@@ -55,6 +55,10 @@ struct Segment {
 // remaining iterations one at a time from the tile's counter, so that a group ends together
 // however its members' speeds differ.  Which iterations land in which partial result then
 // depends on timing: results are reproducible only to rounding.
+// Parts first (split_order != 0; only when every claimer has exactly one range, i.e. without a
+// counter, and runs a whole tile too): a claimer processes its range BEFORE its whole query tile,
+// so that the partial results of the shared tiles are long complete when the workgroups reach
+// their ends and fold them there, a slice each (see fold duties in attn_split.h).
 struct WorkgroupWalk {
   int whole_tile;  // a whole query tile still to do (< 0: none)
   int u_next;      // the range to take next (< 0: none)
@@ -87,7 +91,8 @@ struct WorkgroupWalk {
   // The next segment; false when the workgroup is done.
   template <typename P>
   XDIT_HD bool next(const P& p, int nt, Segment& s) {
-    if (whole_tile >= 0) {
+    const bool range_left = lin < lin_end || (u_next >= 0 && u_next < p.split_units);
+    if (whole_tile >= 0 && !(p.split_order != 0 && range_left)) {
       s.tile = whole_tile; s.it0 = 0; s.it1 = nt; s.slot = -1; s.dyn = -1; s.pool0 = 0;
       whole_tile = -1;
       return true;
@@ -147,6 +152,40 @@ XDIT_HD int shared_tile_parts(const P& p, int nt, int r) {
   const int first_unit = (r * nt) / p.split_len;
   const int last_unit = ((r + 1) * nt - 1) / p.split_len;
   return last_unit - first_unit + 1;
+}
+
+// Folding the parts of a shared query tile inside the attention kernel, without anybody waiting
+// for anybody.  The tile's parts (at most kFoldMaxParts) are folded in slices of rows: slice j,
+// rows [j R / n, (j+1) R / n) of the tile's R rows, is the fold duty of the workgroup that wrote
+// part j of its n parts.  One 32-bit word per shared tile records, through atomic adds only,
+//   bits 0..7    parts that have arrived (partial result written and released),
+//   bits 8..23   slices whose duty was presented before the last part had arrived (deferred),
+//   bits 24..31  events so far: every part contributes two (its arrival and its duty).
+// A workgroup presents its duty either together with its arrival (one add) or later, at its very
+// end (parts-first launches, where the parts are long complete by then).  Whoever makes the tile
+// complete (the last arrival) folds every slice deferred so far (plus its own if it presented its
+// duty with the arrival); a duty presented after completion is folded by its own workgroup.  The
+// atomic adds on one word are totally ordered, so each slice is folded exactly once, after all
+// parts are there; the workgroup that makes the last event puts the word back to zero.
+constexpr int kFoldMaxParts = 16;
+constexpr unsigned kFoldSliceShift = 8, kFoldEventShift = 24;
+XDIT_HD unsigned fold_arrive_word(int j, bool with_duty) {
+  return with_duty ? 1u + (1u << (kFoldSliceShift + j)) + (2u << kFoldEventShift) : 1u + (1u << kFoldEventShift);
+}
+XDIT_HD unsigned fold_duty_word(int j) { return (1u << (kFoldSliceShift + j)) + (1u << kFoldEventShift); }
+// `old` is what the atomic add returned.  The slices (bit j = slice j) to fold now:
+XDIT_HD unsigned fold_after_arrival(unsigned old, int j, bool with_duty, int n) {
+  if ((int)(old & 0xffu) + 1 != n) return 0u;
+  const unsigned deferred = (old >> kFoldSliceShift) & 0xffffu;
+  return with_duty ? deferred | (1u << j) : deferred;
+}
+XDIT_HD unsigned fold_after_duty(unsigned old, int j, int n) { return (int)(old & 0xffu) == n ? 1u << j : 0u; }
+XDIT_HD bool fold_last_event(unsigned old, unsigned word, int n) {
+  return (int)((old >> kFoldEventShift) + (word >> kFoldEventShift)) == 2 * n;
+}
+XDIT_HD void fold_slice_rows(int j, int n, int rows, int& r0, int& r1) {
+  r0 = j * rows / n;
+  r1 = (j + 1) * rows / n;
 }
 
 // Thread -> (row, first 8-element chunk) map of the merge kernel.  A row of `cpr` chunks is held

@@ -66,7 +66,9 @@ struct AttnParams {
                             // streamed sharing: one counter of KV iterations per shared tile
   int split_dyn;      // streamed sharing of the remaining tiles (see WorkgroupWalk)
   int split_s0;       // KV iterations every member of a tile's group owns before it draws from the counter
-  int deterministic;  // fixed work geometry only (no streamed sharing): results reproducible bit for bit
+  int streamed_ok;    // the caller opted in to streamed sharing (results then reproducible to rounding only)
+  int split_order;    // claimers process their range BEFORE their whole query tile (see WorkgroupWalk)
+  int split_fold;     // the parts of a shared tile are folded inside the attention kernel (fold duties, attn_walk.h)
   int split_policy;   // 1: plain launch; 2: balance whenever the plan shortens the critical path by kMinSaving iterations
   // ring step (optional): the result is folded into an fp32 accumulator in the epilogue
   float* acc_out;     // (B,H,Sq,D) fp32 running output, nullptr: plain forward

@@ -67,10 +67,10 @@ _RETIRED = []
 
 
 def _workspace(device, stream, nbytes):
-    """Per-device scratch tensor for balanced launches, grown on demand -> (tensor, preserved).
+    """Per-device scratch tensor for balanced launches, grown on demand -> [tensor, preserved].
     Calls on one stream are ordered, so one buffer per (device, stream) is reused from call to
-    call; nothing else ever writes it, which is what `workspace_preserved` tells the library from
-    the second call on.  A buffer that has become too small is kept alive rather than freed, so
+    call; nothing else ever writes it, which is what `workspace_preserved` tells the library once
+    a call on the buffer has returned without error (the caller sets entry[1] then).  A buffer that has become too small is kept alive rather than freed, so
     that its address cannot come back as a new buffer with foreign contents."""
     key = (device, stream)
     entry = _WORKSPACE.get(key)
@@ -79,16 +79,15 @@ def _workspace(device, stream, nbytes):
             _RETIRED.append(entry[0])
         entry = [torch.empty(int(nbytes), dtype=torch.uint8, device=device), 0]
         _WORKSPACE[key] = entry
-    preserved = entry[1]   # 0 on a buffer's first use: its contents are arbitrary
-    entry[1] = 1
-    return entry[0], preserved
+    return entry   # [tensor, preserved]: preserved is 0 until a call on the buffer has succeeded
 
 
 # Launch tuning passed to the library with every attention call (fields of xdit_attn_args):
 # rows_per_workgroup 0 = the library's choice, else 128 / 256 / 384; cu_count 0 = the device's
 # compute units, else plan the launch as for that many; balance 0 = the library decides whether a
-# launch is balanced, 1 = never, 2 = whenever its planner offers a plan.  Tests and sweeps set these.
-TUNING = {"rows_per_workgroup": 0, "cu_count": 0, "deterministic": 0, "balance": 0}
+# launch is balanced, 1 = never, 2 = whenever its planner offers a plan; streamed 1 = opt in to
+# streamed sharing (results then reproducible to rounding only).  Tests and sweeps set these.
+TUNING = {"rows_per_workgroup": 0, "cu_count": 0, "streamed": 0, "balance": 0}
 
 # Argument structs are filled once per call signature (shapes, strides, dtypes, options) and kept:
 # a later call with the same signature only patches the pointers and the stream.  One set per
@@ -102,10 +101,10 @@ class _AttnPlan:
 
 
 def _sig(t):
-    return None if t is None else (t.shape, t.stride(), t.device)
+    return None if t is None else (t.shape, t.stride(), t.device, t.dtype)
 
 
-def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype, out, lse, acc, deterministic):
+def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype, out, lse, acc, streamed):
     device = q.device
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check4(name, t, device)
@@ -123,7 +122,7 @@ def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype
     a.rows_per_workgroup = int(TUNING["rows_per_workgroup"])
     a.cu_count = int(TUNING["cu_count"])
     a.balance = int(TUNING["balance"])
-    a.deterministic = 1 if deterministic else 0
+    a.streamed_sharing = 1 if streamed else 0
     a.Sq, a.Sk = Sq, k.shape[2]
     a.softmax_scale = float(softmax_scale)
     a.q_stride, a.k_stride, a.v_stride = _strides(q), _strides(k), _strides(v)
@@ -176,18 +175,17 @@ def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype
         r.acc_out_stride = _strides(acc_out)
         r.acc_lse_stride = _lib.Strides(acc_lse.stride(0), acc_lse.stride(1), acc_lse.stride(2))
         plan.ring = r
-    else:
-        with _on_device(device):
-            need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
-        if need < 0:
-            _lib.check(need)
-        plan.need = need
+    with _on_device(device):
+        need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
+    if need < 0:
+        _lib.check(need)
+    plan.need = need
     return plan
 
 
 def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
              q_descale=None, k_descale=None, v_descale=None, out_dtype=None, out=None,
-             return_lse=True, balance=True, lse=None, noalloc=False, deterministic=None, _acc=None):
+             return_lse=True, balance=True, lse=None, noalloc=False, streamed=None, _acc=None):
     """Non-causal attention forward on logical BHSD tensors -> (out BHSD, lse (B,H,Sq) fp32).
 
     `k2`/`v2` are an optional second key/value segment (the joint text tokens) attended together
@@ -195,9 +193,10 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     `out` / `lse` receive the results when given (new tensors otherwise).
     `balance=False` withholds the scratch buffer with which the library evens out the last round
     of workgroups (results then come from one workgroup per query tile).
-    `deterministic=True` asks for results that are reproducible bit for bit from call to call; by
-    default (the reference passes deterministic=False everywhere) a balanced launch may share
-    the KV iterations of a query tile dynamically and results are reproducible to rounding.
+    Results are reproducible bit for bit from call to call, as those of the vendor forwards behind
+    the reference's adapters are; `streamed=True` opts in to a balanced launch that shares the KV
+    iterations of a query tile dynamically (a per cent or two faster on some shapes, results then
+    reproducible to rounding only).
     `noalloc=True` goes through the library's entry point that allocates nothing: the scratch is
     a fixed buffer inside the library (problems that need more than it holds raise ValueError
     unless `balance=False` asks for the plain launch), and `out` (and `lse` when `return_lse`)
@@ -216,17 +215,17 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
         raise ValueError("noalloc needs out (and lse) from the caller and is not available for the ring step")
     if lse is not None:
         return_lse = True
-    if deterministic is None:
-        deterministic = bool(TUNING["deterministic"])
+    if streamed is None:
+        streamed = bool(TUNING["streamed"])
     acc_sig = None if _acc is None else (_sig(_acc[0]), _sig(_acc[1]), _acc[2], _acc[3])
     key = (q.dtype, out_dtype, device, _sig(q), _sig(k), _sig(v), _sig(k2), _sig(v2), _sig(out), _sig(lse),
            k.dtype, v.dtype, float(softmax_scale), bool(causal), q_descale is not None, k_descale is not None,
-           v_descale is not None, acc_sig, TUNING["rows_per_workgroup"], TUNING["cu_count"], TUNING["balance"], bool(deterministic))
+           v_descale is not None, acc_sig, TUNING["rows_per_workgroup"], TUNING["cu_count"], TUNING["balance"], bool(streamed))
     plans = _TLS.__dict__.setdefault("plans", {})
     plan = plans.get(key)
     if plan is None:
         plan = _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, (q_descale, k_descale, v_descale),
-                                out_dtype, out, lse, _acc, deterministic)
+                                out_dtype, out, lse, _acc, streamed)
         if len(plans) >= _PLANS_MAX:
             plans.clear()
         plans[key] = plan
@@ -251,12 +250,9 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
     stream = _stream(device)
     a.stream = stream
     L = _lib.lib()
+    entry = None
     with _on_device(device):
-        if _acc is not None:
-            r = plan.ring
-            r.acc_out, r.acc_lse = _acc[0].data_ptr(), _acc[1].data_ptr()
-            rc = L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r))
-        elif noalloc:
+        if noalloc:
             a.workspace, a.workspace_bytes = None, 0
             if not balance:
                 a.balance = 1   # plain launch: no scratch at all, whatever the size
@@ -264,17 +260,24 @@ def attn_fwd(q, k, v, softmax_scale=None, causal=False, k2=None, v2=None,
             a.balance = int(TUNING["balance"])
         else:
             if balance and plan.need > 0:
-                ws, preserved = _workspace(device, stream, plan.need)
-                a.workspace, a.workspace_bytes, a.workspace_preserved = ws.data_ptr(), ws.numel(), preserved
+                entry = _workspace(device, stream, plan.need)
+                a.workspace, a.workspace_bytes, a.workspace_preserved = entry[0].data_ptr(), entry[0].numel(), entry[1]
             else:
                 a.workspace, a.workspace_bytes, a.workspace_preserved = None, 0, 0
-            rc = L.xdit_attn_fwd(ctypes.byref(a))
+            if _acc is not None:
+                r = plan.ring
+                r.acc_out, r.acc_lse = _acc[0].data_ptr(), _acc[1].data_ptr()
+                rc = L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r))
+            else:
+                rc = L.xdit_attn_fwd(ctypes.byref(a))
+    if entry is not None:
+        entry[1] = 1 if rc == 0 else 0   # after a failure the next call has the counters cleared again
     if rc != 0:
         _lib.check(rc)
     return out, lse
 
 
-def launch_plan(q, k, k2=None, deterministic=None):
+def launch_plan(q, k, k2=None, streamed=None, ring_step=False):
     """How `attn_fwd(q, k, v, k2=..)` would be launched (a dict of the fields of xdit_launch_plan):
     rows per workgroup, query tiles, whole tiles, shared ranges and their length, claimers,
     whether ranges are handed out through the counter, workgroups, workspace bytes.  Host
@@ -289,9 +292,10 @@ def launch_plan(q, k, k2=None, deterministic=None):
     a.rows_per_workgroup = int(TUNING["rows_per_workgroup"])
     a.cu_count = int(TUNING["cu_count"])
     a.balance = int(TUNING["balance"])
-    a.deterministic = 1 if (TUNING["deterministic"] if deterministic is None else deterministic) else 0
+    a.streamed_sharing = 1 if (TUNING["streamed"] if streamed is None else streamed) else 0
     p = _lib.LaunchPlan()
     p.struct_size = ctypes.sizeof(_lib.LaunchPlan)
+    p.ring_step = 1 if ring_step else 0   # the launch of attn_fwd_accumulate instead of attn_fwd's
     _lib.check(_lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)))
     return {name: getattr(p, name) for name, _ in _lib.LaunchPlan._fields_ if name != "struct_size"}
 
@@ -306,7 +310,7 @@ def fused_ring_step_supported(q):
 
 def attn_fwd_accumulate(q, k, v, acc_out, acc_lse, first=False, final_out=None, discard_acc_out=False,
                         softmax_scale=None, k2=None, v2=None, q_descale=None, k_descale=None, v_descale=None,
-                        out_dtype=None):
+                        out_dtype=None, balance=True):
     """One ring step in one launch: attention of q over (k, v) [+ (k2, v2)] folded into the fp32
     accumulator (acc_out logical BHSD, acc_lse logical BHS; any strides) exactly as `attn_fwd`
     followed by `lse_merge` would, without the block ever reaching memory.  `first` initialises
@@ -319,7 +323,7 @@ def attn_fwd_accumulate(q, k, v, acc_out, acc_lse, first=False, final_out=None, 
     if out_dtype is None and final_out is not None:
         out_dtype = final_out.dtype
     attn_fwd(q, k, v, softmax_scale=softmax_scale, k2=k2, v2=v2, out=final_out, return_lse=False,
-             q_descale=q_descale, k_descale=k_descale, v_descale=v_descale, out_dtype=out_dtype,
+             q_descale=q_descale, k_descale=k_descale, v_descale=v_descale, out_dtype=out_dtype, balance=balance,
              _acc=(acc_out, acc_lse, bool(first), bool(discard_acc_out)))
     return acc_out, acc_lse
 
