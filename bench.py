@@ -3,14 +3,19 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
     python bench.py --model-shapes     (a table instead: see below)
-    python bench.py --ceiling-probes   (register-only probes of the matrix pipe, then the Flux step
-                                        on random and on constant inputs: what bounds the kernel)
 
 A "step" is one call of the joint-attention forward on the Flux-1024 shape
 (B=1, H=24, S=4608 = 512 text + 4096 image tokens, D=128, bf16, non-causal, BHSD-contiguous,
-q/k per-head RMSNorm'd), inputs resident in HBM.  Prints ONE JSON line:
+q/k per-head RMSNorm'd), inputs resident in HBM, with the library's default options (fixed work
+geometry: results reproducible bit for bit).  Prints ONE JSON line:
   value        TFLOP/s of the step (algorithmic FLOPs 4*B*H*Sq*Sk*D over wall-clock per step)
-  ms_per_step  wall-clock per call over exactly K calls, synchronised on both sides
+  ms_per_step  wall-clock per call over exactly K calls, synchronised on both sides, after W
+               warm-up calls.  Before the warm-up calls the process brings the chip to its loaded
+               state (`conditioning` in the JSON: about 0.2 s of the same call): coming out of idle
+               the chip's power management lets a few calls run fast, then overshoots downwards
+               for some 100 calls (25 ms) before it settles, and a denoising run, which issues
+               thousands of such calls between GEMMs, lives in the settled state.  The same K calls
+               of a fresh process WITHOUT that conditioning are reported as `also.c2_flux1024_first25`
   roofline     the same kernel's HIP-event average launch duration against the dense bf16 MFMA peak
   cpu_baseline torch's CPU scaled_dot_product_attention (what the reference's SDPA adapter calls,
                xfuser/core/distributed/attention_backend.py:499-501) on a bounded sample of the
@@ -21,7 +26,9 @@ q/k per-head RMSNorm'd), inputs resident in HBM.  Prints ONE JSON line:
                and torch's own GPU flash attention (the op behind the reference's default
                SDPA_FLASH backend, attention_backend.py:504-516) on the same tensors and GPU;
                the PixArt-512 fp32 case; the Flux step's first 25 calls and its steady state in a
-               fresh process (per-call HIP-event pairs: median and min); host time per call
+               fresh process (per-call HIP-event pairs: median and min); the same step with
+               streamed sharing (the opt-in launch whose results are reproducible to rounding
+               only); host time per call
   Entries of `also` carry the median ("ms" / "us"), the minimum and the mean of per-call
   HIP-event pairs (the reference times its own runs with events around synchronised regions
   and discards the first iteration: xfuser/model_executor/models/runner_models/base_model.py:631-644).
@@ -132,22 +139,16 @@ def with_rate(stat, flops, peak=None):
     return stat
 
 
-def series(dev, calls, after_load=False, constant=False):
-    """Per-call HIP-event times (us) of the first `calls` Flux-1024 steps of this process;
-    `after_load`: 150 bf16 matrix products of 8192^3 run first, so that the chip's power
-    management is already in its loaded state when the first step starts; `constant`: q = k = v = 0.5
-    (same launches and traffic, far less switching activity in the matrix pipe)."""
+def _fresh_process_series(calls):
+    """Per-call HIP-event times (us) of the first `calls` Flux-1024 steps of THIS process, printed as
+    one JSON list.  main() runs it in a child process (`python -c "import bench; ..."`), so that the
+    steps are the first GPU work of a process that has just started: no conditioning, no warm-up."""
     from xdit_amd import ops
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
     q, k, v = make_inputs(1, 24, 4608, 128, 1002, dev)
-    if constant:
-        q, k, v = (torch.full_like(t, 0.5) for t in (q, k, v))
     out = torch.empty_like(q)
     lse = torch.empty(1, 24, 4608, dtype=torch.float32, device=dev)
-    if after_load:
-        a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
-        b = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
-        for _ in range(150):
-            torch.matmul(a, b)
     torch.cuda.synchronize()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(calls)]
     for a, b in ev:
@@ -158,23 +159,19 @@ def series(dev, calls, after_load=False, constant=False):
     print(json.dumps([round(a.elapsed_time(b) * 1e3, 1) for a, b in ev]))
 
 
-def data_dependence(dev):
-    """The same launches on random and on constant inputs (steady state, per-call medians): the
-    instructions and the memory traffic are the same, the switching activity of the operands is not."""
-    from xdit_amd import ops
-    for name, (B, H, S) in (("Flux-1024 B=1 H=24 S=4608", (1, 24, 4608)), ("B=1 H=64 S=9216", (1, 64, 9216))):
-        q, k, v = make_inputs(B, H, S, 128, 1002, dev)
-        out = torch.empty_like(q)
-        fl = attn_flops(B, H, S, S, 128)
-        row = []
-        for label, (qq, kk, vv) in (("random q, k, v", (q, k, v)),
-                                    ("q = k = v = 0.5", tuple(torch.full_like(t, 0.5) for t in (q, k, v))),
-                                    ("only k constant", (q, torch.full_like(k, 0.5), v)),
-                                    ("only v constant", (q, k, torch.full_like(v, 0.5))),
-                                    ("only q constant", (torch.full_like(q, 0.5), k, v))):
-            st = time_each(lambda: ops.attn_fwd(qq, kk, vv, out=out), 100, 100)
-            row.append("%s %.1f us = %.0f TFLOP/s" % (label, st["ms"] * 1e3, fl / st["ms"] / 1e9))
-        print("data dependence, %s bf16: %s" % (name, " | ".join(row)), flush=True)
+def condition(fn, seconds=0.2):
+    """Runs `fn` back to back for about `seconds`: the chip's power management is then in the state
+    it keeps under a sustained load of such calls.  Returns the number of calls made."""
+    fn()
+    torch.cuda.synchronize()
+    n = 0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        n += 20
+    return n
 
 
 def attn_flops(B, H, Sq, Sk, D):
@@ -259,15 +256,23 @@ def cpu_baseline(q, k, v, budget_s=8.0):
     q1, k1, v1 = (torch.randn(1, 16, 1024, 72, generator=g) for _ in range(3))
     t1, r1 = _median_time(lambda: O.sdpa_cpu(q1, k1, v1), 1.5, 200)
     others["c1_pixart512_fp32"] = {"s": round(t1, 5), "tflops": round(attn_flops(1, 16, 1024, 1024, 72) / t1 / 1e12, 4), "runs": r1}
-    for name, (Hs, Ss) in (("c4_hunyuan720p_shard", (3, 118800 + 256)), ("c5_wan720p_shard_dequantised_fp32", (5, 75600))):
+    for name, (Hs, Ss, fp8) in (("c4_hunyuan720p_shard", (3, 118800 + 256, False)),
+                                ("c5_wan720p_shard_dequantised_fp32", (5, 75600, True))):
+        # the configurations' own tensors: RMSNorm'd q/k for the HunyuanVideo shard; for the Wan shard
+        # the fp8 tensors with per-head scales, dequantised to fp32 (what an fp32 reference sees)
         rows = 2048
-        qs = torch.randn(1, Hs, rows, D, generator=g)
-        ks, vs = (torch.randn(1, Hs, Ss, D, generator=g) for _ in range(2))
+        cfg = O.make_config("c5_wan720p_shard_fp8" if fp8 else "c4_hunyuan720p_shard")
+        if fp8:
+            qs, ks, vs = (O.dequant(cfg[n], cfg[n + "_descale"]) for n in ("q", "k", "v"))
+        else:
+            qs, ks, vs = (cfg[n].float() for n in ("q", "k", "v"))
+        del cfg
+        qs = qs[:, :, :rows].contiguous()
         ts, rs = _median_time(lambda: O.sdpa_cpu(qs, ks, vs), 2.0, 5)
         others[name] = {"q_rows_measured": rows, "s_measured": round(ts, 4),
                         "tflops": round(attn_flops(1, Hs, rows, Ss, D) / ts / 1e12, 4),
                         "s_whole_shard_extrapolated": round(ts * Ss / rows, 2), "runs": rs,
-                        "note": "fp32, first 2048 query rows x all keys of every shard head; whole-shard time is linear-in-Sq extrapolation, not measured"}
+                        "note": "fp32, first 2048 query rows x all keys of every shard head, the configuration's own tensors; whole-shard time is linear-in-Sq extrapolation, not measured"}
         del qs, ks, vs
     return {
         "value": round(attn_flops(B, H, S, S, D) / t / 1e12, 4),
@@ -291,15 +296,6 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--model-shapes", action="store_true",
                     help="print a table of the reference's model shapes against torch's GPU flash attention, and exit")
-    ap.add_argument("--series", type=int, default=0,
-                    help="print the per-call HIP-event times (us) of the first N Flux-1024 steps of this process, and exit")
-    ap.add_argument("--series-after-load", action="store_true",
-                    help="with --series: run 150 large bf16 matrix products first (the chip is then already under load)")
-    ap.add_argument("--series-constant", action="store_true",
-                    help="with --series: constant inputs (q = k = v = 0.5) instead of the random ones")
-    ap.add_argument("--ceiling-probes", action="store_true",
-                    help="run xdit_amd/csrc/build/mfma_ceiling (MFMA rate on constant and random operands, per-XCD times, "
-                         "MFMA/VALU co-issue), then time the Flux step on random and on constant inputs, and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic for scaling rocprof byte counters)")
     args = ap.parse_args()
@@ -307,15 +303,6 @@ def main():
         print("bench.py: this build runs on ONE GPU only (no collectives / sharding code); --gpus %d is not supported" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
-    if args.ceiling_probes:  # the probe program runs as a child before this process touches the GPU
-        import subprocess
-        exe = os.path.join(ROOT, "xdit_amd", "csrc", "build", "mfma_ceiling")
-        r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
-        sys.stdout.write(r.stdout)
-        sys.stdout.flush()
-        if r.returncode != 0:
-            print("bench.py: %s exited with %d: %s" % (exe, r.returncode, r.stderr[-300:]), file=sys.stderr)
-            sys.exit(1)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
@@ -327,12 +314,6 @@ def main():
     if args.model_shapes:
         model_shapes(dev)
         return
-    if args.series:
-        series(dev, args.series, args.series_after_load, args.series_constant)
-        return
-    if args.ceiling_probes:
-        data_dependence(dev)
-        return
     B, H, S, D = 1, 24, 4608, 128
     q, k, v = make_inputs(B, H, S, D, 1002, dev)
     out = torch.empty_like(q)
@@ -340,12 +321,19 @@ def main():
     def step():
         ops.attn_fwd(q, k, v, out=out)
 
+    conditioning_calls = condition(step, 0.2)
     wall_ms, ev_ms = time_calls(step, args.steps, args.warmup)
     flops = attn_flops(B, H, S, S, D)
     tflops = flops / (wall_ms * 1e-3) / 1e12
     achieved = flops / (ev_ms * 1e-3) / 1e12
 
     traffic, traffic_commit = measured_traffic()
+    plan = ops.launch_plan(q, k)   # what the library launches for this problem
+    kernel_name = "attn_fwd_16_kernel<bf16, head_dim 128, %d wavefronts>: %d query tiles of %d rows, %d whole" % (
+        plan["rows_per_workgroup"] // 32, plan["query_tiles"], plan["rows_per_workgroup"], plan["whole_tiles"])
+    if plan["ranges"]:
+        kernel_name += ", the other %d cut into %d ranges of %d KV iterations%s + attn_combine_kernel<bf16,128>" % (
+            plan["query_tiles"] - plan["whole_tiles"], plan["ranges"], plan["range_len"], " (streamed)" if plan["streamed"] else "")
     result = {
         "metric": "joint-attn fwd ms/call + TFLOP/s (% MFMA peak) at Flux-1024 and HV-720p shard",
         "value": round(tflops, 2),
@@ -363,7 +351,12 @@ def main():
             "workload": "c2_flux1024: joint attention forward (out, lse), B=1 H=24 S=4608 (512 text + 4096 image) D=128, "
                         "bf16, non-causal, BHSD-contiguous, RMSNorm'd q/k, single pass",
             "flops_per_step": flops,
+            "options": "library defaults: fixed work geometry (results reproducible bit for bit); "
+                       "streamed sharing (opt-in) is under also.c2_flux1024_streamed_sharing",
         },
+        "conditioning": "%d untimed calls of the same step over 0.2 s before the %d warm-up calls, so that the chip's power "
+                        "management is in its loaded state; the first calls of a fresh process are under also.c2_flux1024_first25"
+                        % (conditioning_calls, args.warmup),
         "roofline": {
             "bound": "mfma",
             "achieved": round(achieved, 2),
@@ -374,7 +367,7 @@ def main():
             # same counter's reading for a 256 MiB copy in the same run (--copy-calibration)
             "traffic": traffic,
             "traffic_source": "profiles/attn_fwd_bf16_flux1024_hbm_traffic.md, counters taken at commit %s" % traffic_commit,
-            "kernel": "attn_fwd_16_kernel<bf16,128,128,12,false,false> (+ attn_combine_kernel<bf16,128> for the shared last round)",
+            "kernel": kernel_name,
             "kernel_ms": round(ev_ms, 5),
         },
     }
@@ -387,7 +380,8 @@ def main():
         # state (the chip's power management settles), which is where a short timed window lies.
         try:
             import subprocess
-            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--series", "300"], capture_output=True, text=True, timeout=300)
+            r = subprocess.run([sys.executable, "-c", "import bench; bench._fresh_process_series(300)"], cwd=ROOT,
+                               capture_output=True, text=True, timeout=300)
             us = json.loads(r.stdout.strip().splitlines()[-1])
             first, steady = sorted(us[:25]), sorted(us[100:])
             also["c2_flux1024_first25"] = {"us": first[len(first) // 2], "us_min": first[0], "us_max": first[-1],
@@ -402,6 +396,8 @@ def main():
         lse = torch.empty(B, H, S, dtype=torch.float32, device=dev)
         also["host_us_per_call"] = {"attn_fwd": host_us_per_call(lambda: ops.attn_fwd(q, k, v, out=out, lse=lse)),
                                     "attn_fwd_allocating_out_and_lse": host_us_per_call(lambda: ops.attn_fwd(q, k, v))}
+        # the opt-in launch that shares KV iterations of the last round's tiles dynamically (results reproducible to rounding only)
+        also["c2_flux1024_streamed_sharing"] = with_rate(time_each(lambda: ops.attn_fwd(q, k, v, out=out, streamed=True), n, args.warmup), flops, PEAK_BF16_TFLOPS)
         # the plain launch (one workgroup per query tile, no shared last round, no combine kernel)
         also["c2_flux1024_plain_launch"] = with_rate(time_each(lambda: ops.attn_fwd(q, k, v, out=out, balance=False), n, args.warmup), flops)
         # same shape, BSHD-contiguous memory viewed as BHSD (what a single-GPU Flux block hands over)
@@ -421,7 +417,7 @@ def main():
         del q1, k1, v1
         # ring of 4 KV chunks, merged in fp32 (the cast of the last fold is fused)
         fn = usp._get_attention_function()
-        also["c3_flux_ring4"] = with_rate(time_each(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), n, args.warmup), flops)
+        also["c3_flux_ring4"] = with_rate(time_each(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), n, args.warmup), flops, PEAK_BF16_TFLOPS)
         also["host_us_per_call"]["ring4_four_fused_steps"] = host_us_per_call(lambda: usp.ring_attn(fn, q, k, v, ring_chunks=4), batch=10)
         # the same ring captured once in a HIP graph and replayed (shows whether the eager form is launch-bound)
         side = torch.cuda.Stream()
@@ -433,7 +429,7 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             usp.ring_attn(fn, q, k, v, ring_chunks=4)
-        also["c3_flux_ring4_graph"] = with_rate(time_each(graph.replay, n, args.warmup), flops)
+        also["c3_flux_ring4_graph"] = with_rate(time_each(graph.replay, n, args.warmup), flops, PEAK_BF16_TFLOPS)
         del graph
         # the merge kernel alone: bytes per fold = 10*N*D + 12*N
         N = B * H * S

@@ -341,6 +341,30 @@ def test_launch_plan_of_the_named_shapes():
     assert _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(p)) == _lib.XDIT_ERR_UNSUPPORTED
 
 
+def test_launch_choice_against_measured_option_times():
+    """The library's choice of launch (query rows per workgroup, balanced or not) held to
+    measurements: tests/golden/launch_option_times.json records the settled time of every launch
+    option for 180-odd problems on a 256-compute-unit MI355X (16-bit at head_dim 64..128 and fp8;
+    self-attention, ring chunks, cross-attention, long sequences, random shapes).  For every
+    problem the option `xdit_attn_launch_plan` picks (planned for 256 compute units) must be
+    within 15 % of the fastest recorded option, and within 3 % on average per dtype."""
+    import json
+    data = json.load(open(os.path.join(ROOT, "tests", "golden", "launch_option_times.json")))
+    assert len(data["problems"]) > 150
+    loss = {"bf16": [], "fp8": []}
+    for pr in data["problems"]:
+        B, H, Sq, Sk, D = pr["shape"]
+        p = _plan(B, H, Sq, Sk, dtype=_lib.DTYPE_FP8_E4M3FN if pr["dtype"] == "fp8" else None, D=D, cus=data["cu_count"])
+        times = {(rows, bal): t for rows, bal, t in pr["options"]}
+        chosen = (p.rows_per_workgroup, 2 if p.ranges else 1)
+        assert chosen in times, (pr["shape"], chosen)
+        excess = times[chosen] / min(times.values()) - 1.0
+        assert excess <= 0.15, (pr["dtype"], pr["shape"], chosen, times)
+        loss[pr["dtype"]].append(excess)
+    for dtype, xs in loss.items():
+        assert len(xs) > 40 and sum(xs) / len(xs) <= 0.03, (dtype, sum(xs) / len(xs))
+
+
 WALK_HARNESS = r"""
 // Walks every workgroup of a planned launch with the code the kernels run (attn_walk.h) and
 // checks the coverage: stdin holds one launch per line.

@@ -229,6 +229,47 @@ def test_workspace_counters_between_calls(gpu, sharing_mode, force_rows, kind):
     del ops._WORKSPACE[key]
 
 
+def test_workspace_counters_after_a_plain_or_a_failed_first_call(gpu):
+    """`workspace_preserved = 1` is legal after ANY successful call that was given the workspace
+    with 0: a plain launch clears the counters as well (through the C ABI: balance = 1 with a
+    workspace full of ones, then a balanced call that vouches for it).  And the Python wrapper does
+    not vouch for a buffer whose first call failed before anything was launched."""
+    import ctypes
+    g = torch.Generator(device=gpu).manual_seed(9)
+    q, k, v = (torch.randn(1, 3, 4608, 128, generator=g, device=gpu).bfloat16() for _ in range(3))
+    ref_o, ref_l = ops.attn_fwd(q, k, v, balance=False)
+    out, lse = torch.empty_like(q), torch.empty(1, 3, 4608, device=gpu)
+    plan = ops._build_attn_plan(q, k, v, 128 ** -0.5, False, None, None, (None, None, None), q.dtype, out, lse, None, False)
+    assert plan.need > 0
+    a = plan.args
+    a.q, a.k, a.v, a.out, a.lse = (t.data_ptr() for t in (q, k, v, out, lse))
+    a.stream = ops._stream(gpu)
+    ws = torch.full((plan.need,), 0xFF, dtype=torch.uint8, device=gpu)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.workspace_preserved, a.balance = 0, 1          # a plain launch on a fresh workspace
+    assert ops._lib.lib().xdit_attn_fwd(ctypes.byref(a)) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref_o) and int(ws[:16384].max()) == 0 and int(ws[16384:].min()) == 0xFF
+    out.zero_()
+    a.workspace_preserved, a.balance = 1, 0          # then a balanced one that vouches for it
+    assert ops._lib.lib().xdit_attn_fwd(ctypes.byref(a)) == 0
+    torch.cuda.synchronize()
+    assert (out.float() - ref_o.float()).abs().max().item() <= 1e-2 and (lse - ref_l).abs().max().item() <= 1e-5
+    assert int(ws[:16384].max()) == 0
+    # the wrapper: a call that fails validation leaves the buffer unvouched-for
+    key = (q.device, ops._stream(q.device))
+    poisoned = torch.full((plan.need + 64,), 0xFF, dtype=torch.uint8, device=gpu)
+    ops._WORKSPACE[key] = [poisoned, 0]
+    bad_q = torch.empty(q.numel() + 1, dtype=q.dtype, device=gpu)[1:].view(q.shape)   # not 16-byte aligned
+    with pytest.raises(ValueError, match="aligned"):
+        ops.attn_fwd(bad_q, k, v)
+    assert ops._WORKSPACE[key][0] is poisoned and ops._WORKSPACE[key][1] == 0
+    o, l = ops.attn_fwd(q, k, v)
+    assert ops._WORKSPACE[key][1] == 1
+    assert (o.float() - ref_o.float()).abs().max().item() <= 1e-2 and (l - ref_l).abs().max().item() <= 1e-5
+    del ops._WORKSPACE[key]
+
+
 @pytest.fixture
 def force_rows(monkeypatch):
     """Pins the query rows per workgroup (128 / 256 / 384: 4 / 8 / 12 wavefronts) that the library
@@ -1170,6 +1211,55 @@ def test_custom_ops_opcheck_and_compile(gpu):
     e8 = fp8_block(q, k, v)
     c8 = torch.compile(fp8_block, backend="aot_eager", fullgraph=True)(q, k, v)
     assert torch.equal(c8[0], e8[0]) and torch.equal(c8[1], e8[1])
+
+
+def test_custom_ops_ring_step_and_joint_fp8_under_compile(gpu, monkeypatch):
+    """The ring step, the fp8 forward with a second KV segment and the quantiser with a second
+    tensor / a static scale as registered ops: torch's consistency checks, and compiled callers
+    (`torch.compile(fullgraph=True)` of `usp.USP` with joint tensors on the fp8 backend, with a
+    static scale too, and of `usp.ring_attn` over four chunks with joint keys on the last step)
+    give the eager bits without a graph break."""
+    from xdit_amd import custom_ops  # noqa: F401
+    q, k, v = O.make_qkv(1, 2, 512, 128, seed=63, dtype=torch.bfloat16)
+    jq, jk, jv = (t[:, :, :40].contiguous() for t in O.make_qkv(1, 2, 64, 128, seed=64, dtype=torch.bfloat16))
+    q, k, v, jq, jk, jv = (t.to(gpu) for t in (q, k, v, jq, jk, jv))
+    tests = ("test_schema", "test_faketensor", "test_autograd_registration")
+    scale = torch.tensor([0.01], device=gpu)
+    torch.library.opcheck(torch.ops.xdit_amd.fp8_quant_ex.default, (k, jk, None, True, 128), test_utils=tests)
+    torch.library.opcheck(torch.ops.xdit_amd.fp8_quant_ex.default, (k, None, scale, True, 0), test_utils=tests)
+    k8, j8, kd = ops.fp8_quant(k, per_tensor=True, x2=jk)
+    v8, w8, vd = ops.fp8_quant(v, per_tensor=True, x2=jv)
+    q8, qd = ops.fp8_quant(q, per_tensor=True)
+    # (torch's schema check hashes the inputs with arithmetic that fp8 tensors do not have)
+    torch.library.opcheck(torch.ops.xdit_amd.attn_fwd_fp8_joint.default, (q8, k8, v8, j8, w8, qd, kd, vd, 128 ** -0.5, False), test_utils=("test_faketensor", "test_autograd_registration"))
+    acc_o = torch.zeros(1, 2, 512, 128, device=gpu)
+    acc_l = torch.zeros(1, 2, 512, device=gpu)
+    fin = torch.empty_like(q)
+    torch.library.opcheck(torch.ops.xdit_amd.attn_fwd_accumulate.default, (q, k, v, jk, jv, acc_o, acc_l, None, True, False, 128 ** -0.5), test_utils=tests)
+    torch.library.opcheck(torch.ops.xdit_amd.attn_fwd_accumulate.default, (q, k, v, None, None, acc_o, acc_l, fin, False, True, 128 ** -0.5), test_utils=tests)
+
+    def usp_fp8(q, k, v, jq, jk, jv):
+        return usp.USP(q, k, v, joint_query=jq, joint_key=jk, joint_value=jv, joint_strategy="rear",
+                       backend=AB.AttentionBackendType.MI355_FP8)
+
+    eager = usp_fp8(q, k, v, jq, jk, jv)
+    assert torch.equal(torch.compile(usp_fp8, backend="aot_eager", fullgraph=True)(q, k, v, jq, jk, jv), eager)
+    monkeypatch.setattr(AB, "FP8_STATIC_SCALE", 0.02)
+    eager_static = usp_fp8(q, k, v, jq, jk, jv)
+    assert not torch.equal(eager_static, eager)
+    assert torch.equal(torch.compile(usp_fp8, backend="aot_eager", fullgraph=True)(q, k, v, jq, jk, jv), eager_static)
+
+    def ring(q, k, v, jq, jk, jv):
+        return usp.USP(q, k, v, joint_query=jq, joint_key=jk, joint_value=jv, joint_strategy="rear", ring_chunks=4)
+
+    eager_ring = ring(q, k, v, jq, jk, jv)
+    assert torch.equal(torch.compile(ring, backend="aot_eager", fullgraph=True)(q, k, v, jq, jk, jv), eager_ring)
+    fn = usp._get_attention_function()
+
+    def ring_only(q, k, v):
+        return usp.ring_attn(fn, q, k, v, ring_chunks=4)
+
+    assert torch.equal(torch.compile(ring_only, backend="aot_eager", fullgraph=True)(q, k, v), ring_only(q, k, v))
 
 
 # ---------------------------------------------------------------------------- HIP graphs

@@ -142,6 +142,15 @@ def test_custom_ops_fake_implementations_describe_the_outputs():
     assert out.dtype == torch.bfloat16
     y, ds = torch.ops.xdit_amd.fp8_quant(q, False, 128)
     assert y.dtype == torch.float8_e4m3fn and y.shape == q.shape and y.is_contiguous() and ds.shape == (B, H)
+    y, y2, ds = torch.ops.xdit_amd.fp8_quant_ex(k, k2, None, True, 0)
+    assert y.shape == k.shape and y2.shape == k2.shape and y2.dtype == torch.float8_e4m3fn and ds.shape == (B, H)
+    y, y2, ds = torch.ops.xdit_amd.fp8_quant_ex(k, None, torch.empty(1, device="meta"), True, 128)
+    assert y.shape == k.shape and y2.shape == (B, H, 0, D)
+    k28 = torch.empty(B, H, 9, D, dtype=torch.float8_e4m3fn, device="meta")
+    out, lse = torch.ops.xdit_amd.attn_fwd_fp8_joint(q8, k8, k8, k28, k28, d, d, d, 0.1, False)
+    assert out.dtype == torch.bfloat16 and out.shape == (B, H, Sq, D) and lse.shape == (B, H, Sq)
+    acc = torch.empty(B, H, Sq, D, device="meta")
+    assert torch.ops.xdit_amd.attn_fwd_accumulate(q, k, k, k2, k2, acc, torch.empty(B, H, Sq, device="meta"), None, True, False, 0.1) is None
     w = torch.empty(D, dtype=torch.bfloat16, device="meta")
     cs = torch.empty(Sq, D, device="meta")
     y = torch.ops.xdit_amd.norm_rope(q, w, cs, cs, 1e-6, "head", "interleaved", 0, Sq)

@@ -109,19 +109,24 @@ def per_tensor_quant(x, scale=None, scale_dtype=torch.float32, quant_dtype=torch
     concatenated first; the result is then (y, y2, descale)."""
     if quant_dtype != torch.float8_e4m3fn:
         raise NotImplementedError("only float8_e4m3fn (the fp8 format of gfx950) is supported")
-    if scale is None and dtypeMax in (None, get_dtype_max(quant_dtype)):
-        if torch.compiler.is_compiling() and x2 is None:
-            y, descale = torch.ops.xdit_amd.fp8_quant(x, True, hadamard_block)
-            return y, descale.to(scale_dtype)
-        out = ops.fp8_quant(x, per_tensor=True, hadamard_block=hadamard_block, x2=x2)
+    compiling = torch.compiler.is_compiling()   # then through the registered custom ops (fake implementations describe the outputs)
+
+    def quant(scale_tensor):
+        if compiling:
+            y, y2, descale = torch.ops.xdit_amd.fp8_quant_ex(x, x2, scale_tensor, True, hadamard_block)
+            out = (y, descale) if x2 is None else (y, y2, descale)
+        else:
+            out = ops.fp8_quant(x, per_tensor=True, scale=scale_tensor, hadamard_block=hadamard_block, x2=x2)
         return (*out[:-1], out[-1].to(scale_dtype))
+
+    if scale is None and dtypeMax in (None, get_dtype_max(quant_dtype)):
+        return quant(None)
     if scale is None:
         if hadamard_block > 1 or x2 is not None:
             raise NotImplementedError("a non-default dtypeMax together with the fused rotation or a second tensor is not implemented")
         scale = torch.abs(x.to(torch.float32)).max() / dtypeMax
-    scale = torch.as_tensor(scale, dtype=torch.float32, device=x.device)
-    out = ops.fp8_quant(x, per_tensor=True, scale=scale, hadamard_block=hadamard_block, x2=x2)
-    return (*out[:-1], out[-1].to(scale_dtype))
+    scale = torch.as_tensor(scale, dtype=torch.float32, device=x.device).reshape(1)
+    return quant(scale)
 
 
 @register_attention_function(AttentionBackendType.MI355_FP8)
@@ -165,7 +170,9 @@ def _mi355_fp8_attn_call(query, key, value, dropout_p, is_causal, attention_kwar
         v8, v2, vd = per_tensor_quant(value, scale=static, x2=jv)
         if strategy == "front":
             k8, v8, k2, v2 = k2, v2, k8, v8
-    if torch.compiler.is_compiling() and k2 is None:
-        return torch.ops.xdit_amd.attn_fwd_fp8(q8, k8, v8, qd, kd, vd, scale, out_dtype == torch.float16)
+    if torch.compiler.is_compiling():
+        if k2 is None:
+            return torch.ops.xdit_amd.attn_fwd_fp8(q8, k8, v8, qd, kd, vd, scale, out_dtype == torch.float16)
+        return torch.ops.xdit_amd.attn_fwd_fp8_joint(q8, k8, v8, k2, v2, qd, kd, vd, scale, out_dtype == torch.float16)
     return ops.attn_fwd(q8, k8, v8, softmax_scale=scale, k2=k2, v2=v2, q_descale=qd, k_descale=kd, v_descale=vd,
                         out_dtype=out_dtype)

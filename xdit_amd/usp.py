@@ -16,6 +16,7 @@ from . import attention_backend as AB
 from .attention_backend import ATTENTION_FUNCTION_REGISTRY, AttentionBackendType
 
 _DEFAULT_BACKEND = AttentionBackendType.MI355
+_DECORATED = {}   # backend -> (registered function, its joint-decorated wrapper)
 
 
 def set_default_backend(backend):
@@ -48,7 +49,11 @@ def _get_attention_function(backend=None):
     func = ATTENTION_FUNCTION_REGISTRY.get(attention_backend, None)
     if func is None:
         raise NotImplementedError(f"Attention backend {attention_backend} not registered.")
-    return concat_joint_tensors_decorator(func)
+    cached = _DECORATED.get(attention_backend)
+    if cached is None or cached[0] is not func:   # one wrapper per registered function: ring_attn recognises it by identity
+        cached = (func, concat_joint_tensors_decorator(func))
+        _DECORATED[attention_backend] = cached
+    return cached[1]
 
 
 def concat_joint_tensors_decorator(func):
@@ -99,7 +104,13 @@ class SDPAMerger:
         final = None
         if final_step and out.dtype != torch.float32:
             final = torch.empty(out.shape, dtype=out.dtype, device=out.device)
-        ops.lse_merge(self._out, self._lse, out, lse, first=first, final_out=final)
+        if torch.compiler.is_compiling():   # the registered custom ops (traceable)
+            if final is None:
+                torch.ops.xdit_amd.lse_merge(self._out, self._lse, out, lse, first)
+            else:
+                torch.ops.xdit_amd.lse_merge_final(self._out, self._lse, out, lse, final)
+        else:
+            ops.lse_merge(self._out, self._lse, out, lse, first=first, final_out=final)
         self._final = final
 
     def results(self):
@@ -119,9 +130,10 @@ def ring_attn(attention_function, query, key, value, dropout_p=0.0, is_causal=Fa
         order = [0] + list(range(P - 1, 0, -1))
     k_chunks = key.chunk(P, dim=2)
     v_chunks = value.chunk(P, dim=2)
-    base = getattr(attention_function, "__wrapped__", attention_function)
-    if (P > 1 and ops.fused_ring_step_supported(query) and not torch.compiler.is_compiling()
-            and base is ATTENTION_FUNCTION_REGISTRY.get(AttentionBackendType.MI355)):
+    mi355 = ATTENTION_FUNCTION_REGISTRY.get(AttentionBackendType.MI355)
+    decorated = _DECORATED.get(AttentionBackendType.MI355)
+    ours = attention_function is mi355 or (decorated is not None and decorated[0] is mi355 and attention_function is decorated[1])
+    if P > 1 and ops.fused_ring_step_supported(query) and ours:
         # every step is one launch: the kernel folds its block into the accumulator itself (same
         # bits as the call + merge below); the joint keys/values join on the step the decorator
         # would pick
@@ -139,9 +151,13 @@ def ring_attn(attention_function, query, key, value, dropout_p=0.0, is_causal=Fa
                 joint_attn_kwargs["step"] = step + 1
             k1, v1, k2, v2 = AB._split_joint(k_chunks[c], v_chunks[c], joint_kv)
             last = i == P - 1
-            ops.attn_fwd_accumulate(query, k1, v1, acc_out, acc_lse, first=i == 0,
-                                    final_out=final if last else None, discard_acc_out=last,
-                                    softmax_scale=query.shape[-1] ** -0.5, k2=k2, v2=v2)
+            if torch.compiler.is_compiling():   # the same call as a registered custom op (traceable)
+                torch.ops.xdit_amd.attn_fwd_accumulate(query, k1, v1, k2, v2, acc_out, acc_lse, final if last else None,
+                                                       i == 0, last, query.shape[-1] ** -0.5)
+            else:
+                ops.attn_fwd_accumulate(query, k1, v1, acc_out, acc_lse, first=i == 0,
+                                        final_out=final if last else None, discard_acc_out=last,
+                                        softmax_scale=query.shape[-1] ** -0.5, k2=k2, v2=v2)
         return final
     merger = SDPAMerger()
     for i, c in enumerate(order):
