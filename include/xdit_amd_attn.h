@@ -64,7 +64,7 @@ typedef struct {
  * For FP8 inputs q,k,v are multiplied by q_descale[b,h], k_descale[b,h], v_descale[b,h] first.
  * head_dim: a multiple of 8; bf16 / fp16 / fp32 up to 128 (bf16 and fp16 on the 16-bit matrix
  * cores at every such head_dim, at the cost of the next of 64 / 128; fp32 on the fp32 matrix
- * cores), fp8 exactly 128.
+ * cores), fp8 128 or 64.
  * Replaces: attention_backend.py:504-516/:774-823/:887-918 (+ :617-642, :717-772 for fp8) and the
  * kernel call at ring_flash_attn.py:123-134.  The optional second KV segment replaces the
  * torch.cat of joint (text) keys/values at usp.py:239-241 / ring_flash_attn.py:89-100.
@@ -167,7 +167,7 @@ int xdit_attn_fwd_noalloc(const xdit_attn_args* args);
  * c starts with range c and, with counter != 0, takes further ranges from a counter in the
  * workspace.  A query tile's partial results occupy at most `slots_per_tile` workspace slots.
  * bf16 / fp16 (head_dim up to 128; the geometry is that of head_dim 64 or 128, whichever is
- * the next one up) and fp8 (head_dim 128).  fp32 (head_dim up to 128): whole tiles only, of 128
+ * the next one up) and fp8 (head_dim 128 or 64).  fp32 (head_dim up to 128): whole tiles only, of 128
  * rows with `kv_iterations` tiles of 32 keys, or, when those would leave more than a quarter of
  * the compute units without a workgroup, of 64 rows with tiles of 64 keys.  No counterpart in the
  * reference.
@@ -247,7 +247,7 @@ int xdit_lse_merge(const xdit_merge_args* args);
  *                         carry the result); needs args->out
  * acc_out is logical (B,H,Sq,D) fp32, acc_lse logical (B,H,Sq) fp32 with its own strides (the
  * (B,S,H,1) accumulator of the legacy ring maps without a copy).  bf16 / fp16 / fp32 inputs with
- * head_dim a multiple of 8 up to 128, fp8 inputs with head_dim 128; XDIT_ERR_UNSUPPORTED
+ * head_dim a multiple of 8 up to 128, fp8 inputs with head_dim 128 or 64; XDIT_ERR_UNSUPPORTED
  * otherwise (use the two calls).
  * args->workspace (optional, as for xdit_attn_fwd: xdit_attn_workspace_bytes of the same arguments
  * suffices) lets the launch be balanced: the parts of the shared query tiles are then folded and

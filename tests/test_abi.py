@@ -78,7 +78,7 @@ def _attn_args(**kw):
     (dict(rows_per_workgroup=100), _lib.XDIT_ERR_INVALID_ARG, "rows_per_workgroup"),
     (dict(cu_count=-1), _lib.XDIT_ERR_INVALID_ARG, "cu_count"),
     (dict(Sk2=5), _lib.XDIT_ERR_INVALID_ARG, "k2 is NULL"),
-    (dict(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16, D=64), _lib.XDIT_ERR_UNSUPPORTED, "fp8"),
+    (dict(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16, D=96), _lib.XDIT_ERR_UNSUPPORTED, "fp8"),
 ])
 def test_attn_fwd_rejects_bad_arguments(kw, code, needle):
     L = _lib.lib()
@@ -227,7 +227,7 @@ def test_fused_ring_step_rejects_bad_arguments():
     r.acc_out, r.acc_lse = 0x2000, 0x3000
     r.acc_out_stride = _lib.Strides(a.H * a.Sq * a.D, a.Sq * a.D, a.D)
     r.acc_lse_stride = _lib.Strides(a.H * a.Sq, a.Sq, 1)
-    f8 = _attn_args(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16, D=64)  # the fp8 ring step needs head_dim 128
+    f8 = _attn_args(dtype=_lib.DTYPE_FP8_E4M3FN, out_dtype=_lib.DTYPE_BF16, D=32)  # the fp8 ring step needs head_dim 128 or 64
     assert L.xdit_attn_fwd_accumulate(ctypes.byref(f8), ctypes.byref(r)) == _lib.XDIT_ERR_UNSUPPORTED and "fused ring step" in _lib.last_error()
     r.acc_out = 0x2004
     assert L.xdit_attn_fwd_accumulate(ctypes.byref(a), ctypes.byref(r)) == _lib.XDIT_ERR_INVALID_ARG and "acc_out" in _lib.last_error()

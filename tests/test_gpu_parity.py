@@ -500,6 +500,57 @@ def test_fp8_small_vs_oracle(gpu, Sq, Sk):
     assert _err(o, ro) <= 6e-2 * max(1.0, ro.abs().max().item()) and _err(l, rl) <= 1e-3
 
 
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+@pytest.mark.parametrize("rows", [128, 256, 384])
+@pytest.mark.parametrize("Sq,Sk,Sk2", [(1, 1, 0), (100, 63, 0), (129, 130, 50), (300, 1000, 1), (64, 64, 64)])
+def test_fp8_head_dim_64_vs_oracle(gpu, force_rows, layout, rows, Sq, Sk, Sk2):
+    """The fp8 forward at head_dim 64 (SD3, CogVideoX, the audio stream of LTX2: what the
+    reference's hybrid bf16/fp8 schedule hands its fp8 backend for those models): one contraction
+    step of 64 for S^T, two 32-row blocks of O^T.  Every workgroup shape, both memory layouts,
+    ragged sizes and a second KV segment, against the oracle on the dequantised inputs at the
+    absolute 6e-2 / 1e-3 bars."""
+    force_rows(rows)
+    g = torch.Generator().manual_seed(Sq + 7 * Sk + Sk2)
+    q, k, v = (torch.randn(2, 3, n, 64, generator=g) for n in (Sq, Sk + Sk2, Sk + Sk2))
+    (q8, qd), (k8, kd), (v8, vd) = (O.per_head_quant_ref(t) for t in (q, k, v))
+    ro, rl = O.attn_fwd_ref(O.dequant(q8, qd), O.dequant(k8, kd), O.dequant(v8, vd))
+    dev = lambda t: _layout(t.view(torch.uint8), layout, gpu).view(torch.float8_e4m3fn)
+    kw = dict(q_descale=qd.to(gpu), k_descale=kd.to(gpu), v_descale=vd.to(gpu))
+    if Sk2:
+        kw.update(k2=dev(k8[:, :, Sk:].contiguous()), v2=dev(v8[:, :, Sk:].contiguous()))
+    o, l = ops.attn_fwd(dev(q8), dev(k8[:, :, :Sk].contiguous()), dev(v8[:, :, :Sk].contiguous()), **kw)
+    assert o.dtype == torch.bfloat16 and _err(o, ro) <= 6e-2 and _err(l, rl) <= 1e-3
+
+
+def test_fp8_head_dim_64_sd3_shape_balanced_and_ring_step(gpu, monkeypatch):
+    """SD3-1024 joint attention (B=2, H=24, S=4250, head_dim 64) in fp8: the library's launch
+    (balanced) against the plain launch on every row and against the oracle on probe rows; and
+    the fused ring step at head_dim 64 against forward + merge, bit for bit."""
+    g = torch.Generator(device=gpu).manual_seed(64)
+    q, k, v = (torch.randn(2, 24, 4250, 64, generator=g, device=gpu) for _ in range(3))
+    (q8, qd), (k8, kd), (v8, vd) = (ops.fp8_quant(t) for t in (q, k, v))
+    kw = dict(q_descale=qd, k_descale=kd, v_descale=vd)
+    assert ops.launch_plan(q8, k8)["ranges"] > 0
+    o, l = ops.attn_fwd(q8, k8, v8, **kw)
+    po, pl = ops.attn_fwd(q8, k8, v8, balance=False, **kw)
+    assert (o.float() - po.float()).abs().max().item() <= 1e-2 and (l - pl).abs().max().item() <= 1e-5
+    probe = torch.arange(0, 4250, 331)
+    ro, rl = O.attn_fwd_ref(O.dequant(q8.cpu(), qd.cpu())[:, :, probe], O.dequant(k8.cpu(), kd.cpu()), O.dequant(v8.cpu(), vd.cpu()))
+    assert _err(o[:, :, probe.to(gpu)], ro) <= 6e-2 and _err(l[:, :, probe.to(gpu)], rl) <= 1e-3
+    monkeypatch.setitem(ops.TUNING, "streamed", 0)
+    acc_o, acc_l = torch.full((2, 24, 4250, 64), float("nan"), device=gpu), torch.full((2, 24, 4250), float("nan"), device=gpu)
+    ref_o, ref_l = torch.empty_like(acc_o), torch.empty_like(acc_l)
+    fin, ref_fin = torch.empty(2, 24, 4250, 64, dtype=torch.bfloat16, device=gpu), torch.empty(2, 24, 4250, 64, dtype=torch.bfloat16, device=gpu)
+    for i, (a, b) in enumerate(((0, 2000), (2000, 4250))):
+        ks, vs = k8[:, :, a:b], v8[:, :, a:b]
+        ops.attn_fwd_accumulate(q8, ks, vs, acc_o, acc_l, first=i == 0, final_out=fin if i else None, **kw)
+        bo, bl = ops.attn_fwd(q8, ks, vs, **kw)
+        ops.lse_merge(ref_o, ref_l, bo, bl, first=i == 0, final_out=ref_fin if i else None)
+        assert torch.equal(acc_o, ref_o) and torch.equal(acc_l, ref_l), i
+    assert torch.equal(fin, ref_fin)
+    assert (fin.float() - o.float()).abs().max().item() <= 2e-2 and (acc_l - l).abs().max().item() <= 1e-4   # two chunks = single pass
+
+
 @pytest.mark.parametrize("balance", [1, 2])
 @pytest.mark.parametrize("rows", [128, 256, 384])
 @pytest.mark.parametrize("kind,D", [("bf16", 128), ("bf16", 64), ("fp16", 96), ("fp8", 128)])

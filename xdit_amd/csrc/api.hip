@@ -275,8 +275,8 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   if (acc != nullptr) {
     if (acc->struct_size != sizeof(xdit_ring_acc))
       return fail(XDIT_ERR_INVALID_ARG, "acc struct_size %u != %zu (ABI mismatch)", acc->struct_size, sizeof(xdit_ring_acc));
-    if (a->dtype == XDIT_DTYPE_FP8_E4M3FN ? a->D != 128 : a->D > 128)
-      return fail(XDIT_ERR_UNSUPPORTED, "the fused ring step needs head_dim at most 128 (fp8: 128), got %d", a->D);
+    if (a->dtype == XDIT_DTYPE_FP8_E4M3FN ? (a->D != 128 && a->D != 64) : a->D > 128)
+      return fail(XDIT_ERR_UNSUPPORTED, "the fused ring step needs head_dim at most 128 (fp8: 128 or 64), got %d", a->D);
     if ((rc = check_tensor("acc_out", acc->acc_out, acc->acc_out_stride, 4, a->D))) return rc;
     if (acc->acc_lse == nullptr) return fail(XDIT_ERR_INVALID_ARG, "acc_lse is NULL");
     if (acc->acc_lse_stride.b < 0 || acc->acc_lse_stride.h < 0 || acc->acc_lse_stride.s <= 0)
@@ -319,14 +319,14 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
   hipStream_t stream = (hipStream_t)a->stream;
 
   const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN;
-  if (fp8 && a->D != 128) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 only (got %d)", a->D);
+  if (fp8 && a->D != 128 && a->D != 64) return fail(XDIT_ERR_UNSUPPORTED, "fp8 attention supports head_dim 128 and 64 only (got %d)", a->D);
   if (!fp8 && !mfma16_path(a) && a->D > 128) return fail(XDIT_ERR_UNSUPPORTED, "head_dim %d above 128 is not implemented", a->D);
   // A workspace whose contents the caller does not vouch for gets its counters cleared, whatever
   // launch follows: the next call on it may then say "preserved" whether this one is balanced or not.
   if (p.ws_out != nullptr && !p.ws_preserved) xdit::launch_counter_reset(p.ws_out, stream);
   hipError_t e;
   if (fp8 || mfma16_path(a)) {
-    const int D = fp8 ? 128 : kernel_head_dim(a->D);
+    const int D = fp8 ? a->D : kernel_head_dim(a->D);
     if (!fp8) p.d_actual = a->D;
     const bool fused = acc != nullptr;
     LaunchChoice c = choose_launch(a, p.ws_out == nullptr, fused);  // no workspace: the shape that suits a plain launch
@@ -334,13 +334,13 @@ static int attn_fwd_impl(const xdit_attn_args* a, const xdit_ring_acc* acc) {
     if (c.policy == 2) {
       // a workspace too small for the chosen balanced plan: the best PLAIN launch, not that shape run plain
       xdit::AttnParams plan;
-      const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, c.rows, &plan, fused) : xdit::attn_fwd_16_workspace(p, D, c.rows, &plan, fused);
+      const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, D, c.rows, &plan, fused) : xdit::attn_fwd_16_workspace(p, D, c.rows, &plan, fused);
       if (need > p.ws_bytes) {
         c = choose_launch(a, true, fused);
         p.split_policy = c.policy;
       }
     }
-    if (fp8) e = xdit::launch_attn_fwd_fp8(p, out_dtype == XDIT_DTYPE_FP16, c.rows, stream);
+    if (fp8) e = xdit::launch_attn_fwd_fp8(p, D, out_dtype == XDIT_DTYPE_FP16, c.rows, stream);
     else e = fused ? xdit::launch_attn_fwd_16_ring(p, a->dtype == XDIT_DTYPE_FP16, D, c.rows, stream)
                    : xdit::launch_attn_fwd_16(p, a->dtype == XDIT_DTYPE_FP16, D, c.rows, stream);
   } else {
@@ -412,10 +412,10 @@ int64_t xdit_attn_workspace_bytes(const xdit_attn_args* a) {
   p.B = a->B; p.H = a->H; p.Sq = (int)a->Sq; p.Sk = (int)a->Sk; p.Sk2 = (int)a->Sk2;
   p.cu_count = a->cu_count;
   p.streamed_ok = a->streamed_sharing != 0;
-  if (!(a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128) && !mfma16_path(a)) return 0;
+  if (!(a->dtype == XDIT_DTYPE_FP8_E4M3FN && (a->D == 128 || a->D == 64)) && !mfma16_path(a)) return 0;
   const LaunchChoice c = choose_launch(a);
   p.split_policy = c.policy;
-  if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) return (int64_t)xdit::attn_fwd_fp8_workspace(p, c.rows);
+  if (a->dtype == XDIT_DTYPE_FP8_E4M3FN) return (int64_t)xdit::attn_fwd_fp8_workspace(p, a->D, c.rows);
   return (int64_t)xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), c.rows);
 }
 
@@ -431,7 +431,7 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
       (int64_t)a->B * a->H * ((a->Sq + 31) / 32) > (int64_t(1) << 30))
     return fail(XDIT_ERR_INVALID_ARG, "bad shape");
   if (int rc0 = check_tuning(a)) return rc0;
-  const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN && a->D == 128;
+  const bool fp8 = a->dtype == XDIT_DTYPE_FP8_E4M3FN && (a->D == 128 || a->D == 64);
   const bool b16 = mfma16_path(a);
   xdit::AttnParams p, q;
   std::memset(&p, 0, sizeof(p));
@@ -457,7 +457,7 @@ int xdit_attn_launch_plan(const xdit_attn_args* a, xdit_launch_plan* out) {
   const LaunchChoice choice = choose_launch(a, false, ring_step);
   const int rows = choice.rows;
   p.split_policy = choice.policy;
-  const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, rows, &q, ring_step) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q, ring_step);
+  const size_t need = fp8 ? xdit::attn_fwd_fp8_workspace(p, a->D, rows, &q, ring_step) : xdit::attn_fwd_16_workspace(p, kernel_head_dim(a->D), rows, &q, ring_step);
   const uint32_t size = out->struct_size;
   std::memset(out, 0, sizeof(*out));
   out->struct_size = size;

@@ -1,10 +1,11 @@
 // Non-causal attention forward for fp8 (OCP e4m3fn) Q/K/V with per-(batch, head) fp32 descales,
-// head_dim 128, bf16 or fp16 output, fp32 log-sum-exp, on gfx950.
+// head_dim 128 or 64, bf16 or fp16 output, fp32 log-sum-exp, on gfx950.
 //
 // Same structure as the 16-bit kernel (workgroup = 4, 8 or 12 wavefronts x 32 query rows, 64-key
 // K/V tiles double buffered in LDS by direct global->LDS loads, hand-issued LDS fragment reads,
 // transposed products so that each lane owns one query), with v_mfma_f32_32x32x64_f8f6f4 for both products:
-//   S^T = K Q^T    A = K rows, B = Q^T (registers); contraction over head_dim, 64 per instruction.
+//   S^T = K Q^T    A = K rows, B = Q^T (registers); contraction over head_dim, 64 per instruction
+//                  (two steps at head_dim 128, one at 64).
 //                  A and B use the same lane->contraction-index map, so each lane simply holds the
 //                  32 contiguous bytes d = 64ks + 32(l/32) .. +31 of its row.
 //   O^T = V^T P^T  contraction over the 64 keys of the tile in ONE instruction per 32 rows of
@@ -24,20 +25,25 @@ namespace xdit {
 namespace fp8path {
 
 constexpr int kRowsPerWave = 32;
-constexpr int D = 128;
 constexpr float kPShift = 6.0f;           // P is scaled by 2^6 ...
 constexpr float kLazyRescaleLog2 = 2.0f;  // ... and the row max may lag by 2^2: P <= 2^8 < 448
 
-// LDS tile geometry: rows of 128 bytes, 8 rows per 1 KiB piece, 8 pieces per 64-key tile;
-// row r lives in piece r % 8 at slot r / 8.  Piece pitches pad by 16 B (K: 16-byte reads of 16
-// consecutive rows) and 32 B (V: 32-byte row segments of 8 rows) to spread the banks.
-constexpr int ROW_BYTES = 128;
-constexpr int NG = 8;
-constexpr int K_PITCH = 1024 + 16;
-constexpr int V_PITCH = 1024 + 32;
-constexpr int K_BYTES = NG * K_PITCH;
-constexpr int V_BYTES = NG * V_PITCH;
-constexpr int BUF_BYTES = K_BYTES + V_BYTES;
+// LDS tile geometry: rows of D bytes, 1024 / D rows per 1 KiB piece (what one wavefront
+// instruction of the direct global->LDS load writes), NG pieces per 64-key tile; row r lives in
+// piece r % NG at slot r / NG.  Piece pitches pad by 16 B (K: 16-byte reads of consecutive rows)
+// and 32 B (V: 32-byte row segments) to spread the banks.
+template <int D> struct Geom {
+  static_assert(D == 128 || D == 64, "head_dim of the fp8 kernels");
+  static constexpr int ROW_BYTES = D;
+  static constexpr int NG = kKeysPerTile * D / 1024;   // 8 or 4
+  static constexpr int K_PITCH = 1024 + 16;
+  static constexpr int V_PITCH = 1024 + 32;
+  static constexpr int K_BYTES = NG * K_PITCH;
+  static constexpr int V_BYTES = NG * V_PITCH;
+  static constexpr int BUF_BYTES = K_BYTES + V_BYTES;
+  static constexpr int KS = D / 64;   // contraction steps of S^T
+  static constexpr int DB = D / 32;   // 32-row blocks of O^T
+};
 // LDS fragment reads are issued this many MFMAs ahead of the MFMA that consumes them.
 constexpr int kPrefetch = 2;
 
@@ -47,8 +53,8 @@ constexpr int kStagePitch = 64 * 2 + 8;
 constexpr int kStageBytes = kRowsPerWave * kStagePitch + kRowsPerWave * 4;  // + one fp32 per row (ring step)
 // LDS of a workgroup: the first K/V buffer, then a region that holds the second K/V buffer during
 // the KV loop and the output staging blocks of the wavefronts in the epilogue.
-template <int NW>
-constexpr int lds_bytes() { return BUF_BYTES + (BUF_BYTES > NW * kStageBytes ? BUF_BYTES : NW * kStageBytes); }
+template <int D, int NW>
+constexpr int lds_bytes() { return Geom<D>::BUF_BYTES + (Geom<D>::BUF_BYTES > NW * kStageBytes ? Geom<D>::BUF_BYTES : NW * kStageBytes); }
 
 // The work of one workgroup: its segments (WorkgroupWalk), one after the other; a segment is the
 // query tile `tile` and KV tiles [it0, it1), written to the output tensors (slot < 0) or as one
@@ -61,9 +67,12 @@ constexpr int lds_bytes() { return BUF_BYTES + (BUF_BYTES > NW * kStageBytes ? B
 // folded into the fp32 accumulator with the arithmetic of the merge kernel, so that the result
 // equals forward + merge bit for bit; the parts of shared tiles go through the workspace as in a plain
 // forward and are folded, then folded into the accumulator, by the fold duties.
-template <typename TO, int NW, bool FUSED>
+template <typename TO, int D, int NW, bool FUSED>
 __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
   typedef unsigned char u8;
+  typedef Geom<D> G;
+  constexpr int ROW_BYTES = G::ROW_BYTES, NG = G::NG, K_PITCH = G::K_PITCH, V_PITCH = G::V_PITCH, K_BYTES = G::K_BYTES,
+                BUF_BYTES = G::BUF_BYTES, KS = G::KS, DB = G::DB;
   ParamsPtr pp = (ParamsPtr)__builtin_amdgcn_kernarg_segment_ptr();
   constexpr int kWaves = NW;
   constexpr int kRowsPerBlock = kRowsPerWave * kWaves;
@@ -86,10 +95,11 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
   // ---- tile loads ------------------------------------------------------------------------
   // Loader wavefronts: the first LW wavefronts each load PAIRS (K piece g, V piece g) pairs,
   // g = wave + LW * i, with one row index per lane for both pieces of a pair.
-  constexpr int LW = kWaves < 8 ? kWaves : 8;
+  constexpr int LW = kWaves < NG ? kWaves : NG;
   constexpr int PAIRS = NG / LW;
-  int ld_row0 = NG * (lane >> 3) + wave;    // 8 lanes per 128-byte row: row of this lane in pair 0
-  unsigned ld_colb = (lane & 7) * 16;
+  constexpr int LANES_PER_ROW = ROW_BYTES / 16;
+  int ld_row0 = NG * (lane / LANES_PER_ROW) + wave;    // row of this lane in pair 0
+  unsigned ld_colb = (lane % LANES_PER_ROW) * 16;
   asm volatile("" : "+v"(ld_row0), "+v"(ld_colb));
   const unsigned lds_base = (unsigned)(uintptr_t)(XDIT_LDS u8*)smem;
   const unsigned ld_kdst = lds_base + wave * K_PITCH;  // LDS address of K piece `wave`, buffer 0
@@ -124,20 +134,23 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
 
   // ---- LDS read bases ------------------------------------------------------------------------
   // K fragment for key block kb, step ks: row 32kb + l32, bytes 64ks + 32hh .. +31.
-  unsigned kbase_off = lds_base + (l32 & 7) * K_PITCH + (l32 >> 3) * ROW_BYTES + hh * 32;
+  unsigned kbase_off = lds_base + (l32 % NG) * K_PITCH + (l32 / NG) * ROW_BYTES + hh * 32;
+  constexpr int K_KB_STEP = (32 / NG) * ROW_BYTES;   // +32 rows = +32/NG slots
   // V^T fragment, read r (0..3), d block db: as a SOURCE lane of ds_read_b64_tr_b8, lane
   // (group g = lane/16, s = lane%16) supplies 8 bytes of key row 16r + 8(s/8) + 4hh + (s/2)%4
   // at d = 32db + 16(g%2) + 8(s%2); lane (g, i) receives d = 32db + 16(g%2) + i for the 8 keys
   // 16r + 8(j/4) + 4hh + j%4, j = 0..7.
   const int s16 = lane & 15;
-  unsigned vbase_off = lds_base + K_BYTES + (4 * hh + ((s16 >> 1) & 3)) * V_PITCH + (s16 >> 3) * ROW_BYTES +
+  const int vrow0 = 8 * (s16 >> 3) + 4 * hh + ((s16 >> 1) & 3);   // key row of read 0; read r is 16 r further
+  unsigned vbase_off = lds_base + K_BYTES + (vrow0 % NG) * V_PITCH + (vrow0 / NG) * ROW_BYTES +
                        16 * ((lane >> 4) & 1) + 8 * (s16 & 1);
+  constexpr int V_R_STEP = (16 / NG) * ROW_BYTES;    // +16 rows
   asm volatile("" : "+v"(kbase_off), "+v"(vbase_off));  // one register each through the loop
 
   // ---- per segment: coordinates, Q fragments (2 contraction steps x 32 bytes), scales, first tile
   int b, h, qt;
   float c, sv;
-  i32x8 qf[2];
+  i32x8 qf[KS];
   auto open_segment = [&](const Segment& sg) {
     const int lane = lane_now(), l32 = lane & 31, hh = lane >> 5;
     const int nq_tiles = pp->nq_tiles, H = pp->H;
@@ -168,7 +181,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
     const int qrow_c = qrow < Sq ? qrow : Sq - 1;
     const u8* qptr = (const u8*)pp->q + b * pp->qs_b + h * pp->qs_h + (int64_t)qrow_c * pp->qs_s + hh * 32;
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
+    for (int ks = 0; ks < KS; ks++) {
       i32x4 lo = *(const i32x4*)(qptr + ks * 64);
       i32x4 hi = *(const i32x4*)(qptr + ks * 64 + 16);
       qf[ks] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -188,13 +201,13 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
     const int keys_1 = keys1, keys_2 = keys2;
     float m_used = -INFINITY;
     float l_part = 0.f;
-    f32x16 oacc[4];
+    f32x16 oacc[DB];
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < DB; db++)
 #pragma unroll
       for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++) asm volatile("" : "+v"(qf[ks]));
+    for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));
 
     for (int t = seg.it0; t < seg.it1; t++) {
       const int buf = (t - seg.it0) & 1;
@@ -206,16 +219,16 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
       const unsigned vaddr = vbase_off + buf * BUF_BYTES;
 
       // ---- S^T = K Q^T ---------------------------------------------------------------------
-      // Four MFMAs; MFMA m = 2 ks + kb (consecutive ones share their Q fragment) takes the 32 bytes
+      // 2 KS MFMAs; MFMA m = 2 ks + kb (consecutive ones share their Q fragment) takes the 32 bytes
       // of its K row as two 16-byte reads.
       f32x16 sacc[2];
       {
         constexpr int PD = kPrefetch;  // MFMAs whose two reads are in flight
-        constexpr int NM = 4;
+        constexpr int NM = 2 * KS;
         i32x4 klo[NM], khi[NM];
         static_for<PD>([&](auto I) {
           constexpr int m = I;
-          constexpr int off = (m % 2) * 4 * ROW_BYTES + (m / 2) * 64;
+          constexpr int off = (m % 2) * K_KB_STEP + (m / 2) * 64;
           lds_read_b128<off>(klo[m], kaddr);
           lds_read_b128<off + 16>(khi[m], kaddr);
         });
@@ -231,7 +244,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
           sacc[m % 2] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf[m / 2], sacc[m % 2], 0, 0, 0, 0, 0, 0);
           if constexpr (m + PD < NM) {
             constexpr int n = m + PD;
-            constexpr int off = (n % 2) * 4 * ROW_BYTES + (n / 2) * 64;
+            constexpr int off = (n % 2) * K_KB_STEP + (n / 2) * 64;
             lds_read_b128<off>(klo[n], kaddr);
             lds_read_b128<off + 16>(khi[n], kaddr);
           }
@@ -264,7 +277,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
         m_used = m_new;
         l_part *= alpha;
 #pragma unroll
-        for (int db = 0; db < 4; db++)
+        for (int db = 0; db < DB; db++)
 #pragma unroll
           for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
       }
@@ -288,16 +301,16 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
       }
 
       // ---- O^T += V^T P^T ------------------------------------------------------------------
-      // Four MFMAs (d blocks); each takes its V^T operand as four transposing 8-byte reads.
+      // One MFMA per d block; each takes its V^T operand as four transposing 8-byte reads.
       {
         constexpr int PD = kPrefetch;
-        constexpr int NM = 4;
+        constexpr int NM = DB;
         i32x2 vr[NM][4];
         static_for<PD>([&](auto I) {
           constexpr int m = I;
           static_for<4>([&](auto R) {
             constexpr int r = R;
-            lds_read_tr8_b64<r * 2 * ROW_BYTES + m * 32>(vr[m][r], vaddr);
+            lds_read_tr8_b64<r * V_R_STEP + m * 32>(vr[m][r], vaddr);
           });
         });
         static_for<NM>([&](auto I) {
@@ -315,7 +328,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
             constexpr int n = m + PD;
             static_for<4>([&](auto R) {
               constexpr int r = R;
-              lds_read_tr8_b64<r * 2 * ROW_BYTES + n * 32>(vr[n][r], vaddr);
+              lds_read_tr8_b64<r * V_R_STEP + n * 32>(vr[n][r], vaddr);
             });
           }
         });
@@ -365,7 +378,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
       const int rd_row = lane >> 3;          // + 8r
       const int rd_col = (lane & 7) * 8;     // element column within the 64-column pass
 #pragma unroll
-      for (int half = 0; half < 2; half++) {
+      for (int half = 0; half < D / 64; half++) {
 #pragma unroll
         for (int dbl = 0; dbl < 2; dbl++) {
           const int db = 2 * half + dbl;
@@ -413,7 +426,7 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
       const int rd_row = lane >> 3;
       const int rd_col = (lane & 7) * 8;
 #pragma unroll
-      for (int half = 0; half < 2; half++) {
+      for (int half = 0; half < D / 64; half++) {
 #pragma unroll
         for (int dbl = 0; dbl < 2; dbl++) {
           const int db = 2 * half + dbl;
@@ -478,16 +491,16 @@ __device__ __forceinline__ void attn_workgroup_fp8(unsigned char* smem) {
   }
 }
 
-template <typename TO, int NW, bool FUSED>
+template <typename TO, int D, int NW, bool FUSED>
 __global__ __launch_bounds__(64 * NW, NW == 8 ? 2 : 3) void attn_fwd_fp8_kernel(const AttnParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // [K tile | V tile] [K tile | V tile, or output staging]
-  attn_workgroup_fp8<TO, NW, FUSED>(smem);
+  attn_workgroup_fp8<TO, D, NW, FUSED>(smem);
 }
 
 // Workgroups of NW wavefronts resident at once (3 wavefronts per SIMD by registers; 2 for NW = 8).
 static int resident_workgroups(int NW, int planned_cus) { return resident_cus(planned_cus) * (NW == 4 ? 3 : 1); }
 
-template <typename TO, int NW, bool FUSED>
+template <typename TO, int D, int NW, bool FUSED>
 static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   AttnParams q = p;
   constexpr int rows = kRowsPerWave * NW;
@@ -497,15 +510,15 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   // the ring step takes a balanced plan only when the attention kernel folds the parts itself (the fold goes on into the accumulator)
   bind_workspace(q, p, plan_split(q, rows, resident_workgroups(NW, p.cu_count), D, 2, 1, false, FUSED), rows, D, 2);
   static std::atomic<bool> lds_ready[kMaxDevices];
-  constexpr int lds = lds_bytes<NW>();
+  constexpr int lds = lds_bytes<D, NW>();
   const int slot = current_device_slot();
   if (lds > 65536 && !lds_ready[slot].load(std::memory_order_relaxed)) {  // > 64 KiB of dynamic LDS must be enabled once per kernel and device
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_fp8_kernel<TO, NW, FUSED>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_fp8_kernel<TO, D, NW, FUSED>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     lds_ready[slot].store(true, std::memory_order_relaxed);
   }
   dim3 grid(split_grid(q));
-  hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, NW, FUSED>), grid, dim3(64 * NW), lds, stream, q);
+  hipLaunchKernelGGL((attn_fwd_fp8_kernel<TO, D, NW, FUSED>), grid, dim3(64 * NW), lds, stream, q);
   if constexpr (!FUSED) {
     if (q.split_units && !q.split_fold) {  // tiles of many parts: folded by a launch of its own
       const int nt = (q.Sk + kKeysPerTile - 1) / kKeysPerTile + (q.Sk2 + kKeysPerTile - 1) / kKeysPerTile;
@@ -516,7 +529,7 @@ static hipError_t launch_one(const AttnParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int NW>
+template <int D, int NW>
 static size_t workspace_one(const AttnParams& p, AttnParams* plan, bool fold_only) {
   AttnParams q = p;
   constexpr int rows = kRowsPerWave * NW;
@@ -531,24 +544,31 @@ static size_t workspace_one(const AttnParams& p, AttnParams* plan, bool fold_onl
 }  // namespace fp8path
 
 // rows_per_block: 128 (4 wavefronts), 256 (8) or 384 (12 wavefronts sharing each K/V tile).
-template <bool FUSED>
+template <int D, bool FUSED>
 static hipError_t launch_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream) {
   using namespace fp8path;
-  if (rows_per_block == 384) return out_is_fp16 ? launch_one<_Float16, 12, FUSED>(p, stream) : launch_one<__bf16, 12, FUSED>(p, stream);
-  if (rows_per_block == 256) return out_is_fp16 ? launch_one<_Float16, 8, FUSED>(p, stream) : launch_one<__bf16, 8, FUSED>(p, stream);
-  return out_is_fp16 ? launch_one<_Float16, 4, FUSED>(p, stream) : launch_one<__bf16, 4, FUSED>(p, stream);
+  if (rows_per_block == 384) return out_is_fp16 ? launch_one<_Float16, D, 12, FUSED>(p, stream) : launch_one<__bf16, D, 12, FUSED>(p, stream);
+  if (rows_per_block == 256) return out_is_fp16 ? launch_one<_Float16, D, 8, FUSED>(p, stream) : launch_one<__bf16, D, 8, FUSED>(p, stream);
+  return out_is_fp16 ? launch_one<_Float16, D, 4, FUSED>(p, stream) : launch_one<__bf16, D, 4, FUSED>(p, stream);
 }
 
-// p.acc_out set: the ring step (fold into the fp32 accumulator in the epilogue).
-hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream) {
-  return p.acc_out != nullptr ? launch_fp8<true>(p, out_is_fp16, rows_per_block, stream) : launch_fp8<false>(p, out_is_fp16, rows_per_block, stream);
+// D: 128 or 64.  p.acc_out set: the ring step (fold into the fp32 accumulator in the epilogue).
+hipError_t launch_attn_fwd_fp8(const AttnParams& p, int D, int out_is_fp16, int rows_per_block, hipStream_t stream) {
+  if (D == 128) return p.acc_out != nullptr ? launch_fp8<128, true>(p, out_is_fp16, rows_per_block, stream) : launch_fp8<128, false>(p, out_is_fp16, rows_per_block, stream);
+  if (D == 64) return p.acc_out != nullptr ? launch_fp8<64, true>(p, out_is_fp16, rows_per_block, stream) : launch_fp8<64, false>(p, out_is_fp16, rows_per_block, stream);
+  return hipErrorInvalidValue;
 }
 
-size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan, bool fold_only) {
+size_t attn_fwd_fp8_workspace(const AttnParams& p, int D, int rows_per_block, AttnParams* plan, bool fold_only) {
   using namespace fp8path;
-  if (rows_per_block == 384) return workspace_one<12>(p, plan, fold_only);
-  if (rows_per_block == 256) return workspace_one<8>(p, plan, fold_only);
-  return workspace_one<4>(p, plan, fold_only);
+  if (D == 128) {
+    if (rows_per_block == 384) return workspace_one<128, 12>(p, plan, fold_only);
+    if (rows_per_block == 256) return workspace_one<128, 8>(p, plan, fold_only);
+    return workspace_one<128, 4>(p, plan, fold_only);
+  }
+  if (rows_per_block == 384) return workspace_one<64, 12>(p, plan, fold_only);
+  if (rows_per_block == 256) return workspace_one<64, 8>(p, plan, fold_only);
+  return workspace_one<64, 4>(p, plan, fold_only);
 }
 
 }  // namespace xdit

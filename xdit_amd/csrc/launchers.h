@@ -79,8 +79,8 @@ struct PrologueBatch {
 hipError_t launch_attn_fwd_16(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream);
 hipError_t launch_attn_fwd_16_ring(const AttnParams& p, int dtype_is_fp16, int D, int rows_per_block, hipStream_t stream);  // p.acc_out set
 size_t attn_fwd_16_workspace(const AttnParams& p, int D, int rows_per_block, AttnParams* plan = nullptr, bool fold_only = false);  // fold_only: the ring step
-hipError_t launch_attn_fwd_fp8(const AttnParams& p, int out_is_fp16, int rows_per_block, hipStream_t stream);
-size_t attn_fwd_fp8_workspace(const AttnParams& p, int rows_per_block, AttnParams* plan = nullptr, bool fold_only = false);
+hipError_t launch_attn_fwd_fp8(const AttnParams& p, int D, int out_is_fp16, int rows_per_block, hipStream_t stream);  // D: 128 or 64
+size_t attn_fwd_fp8_workspace(const AttnParams& p, int D, int rows_per_block, AttnParams* plan = nullptr, bool fold_only = false);
 hipError_t launch_attn_fwd_f32(const AttnParams& p, int D, hipStream_t stream);  // fp32 tensors only
 int attn_fwd_f32_rows(const AttnParams& p);  // query rows per workgroup the fp32 launch takes: 128, or 64 (64-key tiles split between wavefront pairs)
 hipError_t launch_fp8_quant(const QuantParams& p, int in_dtype, hipStream_t stream);

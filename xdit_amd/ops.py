@@ -281,7 +281,7 @@ def launch_plan(q, k, k2=None, streamed=None, ring_step=False):
     """How `attn_fwd(q, k, v, k2=..)` would be launched (a dict of the fields of xdit_launch_plan):
     rows per workgroup, query tiles, whole tiles, shared ranges and their length, claimers,
     whether ranges are handed out through the counter, workgroups, workspace bytes.  Host
-    arithmetic only; bf16 / fp16 / fp32 (head_dim up to 128) and fp8 (head_dim 128)."""
+    arithmetic only; bf16 / fp16 / fp32 (head_dim up to 128) and fp8 (head_dim 128 or 64)."""
     a = _lib.AttnArgs()
     a.struct_size = ctypes.sizeof(_lib.AttnArgs)
     a.dtype = _code(q.dtype)
@@ -302,9 +302,9 @@ def launch_plan(q, k, k2=None, streamed=None, ring_step=False):
 
 def fused_ring_step_supported(q):
     """Whether `attn_fwd_accumulate` takes these queries (bf16 / fp16 / fp32 with head_dim a multiple
-    of 8 up to 128, fp8 with head_dim 128)."""
+    of 8 up to 128, fp8 with head_dim 128 or 64)."""
     if q.dtype == torch.float8_e4m3fn:
-        return q.shape[-1] == 128
+        return q.shape[-1] in (128, 64)
     return q.dtype in (torch.bfloat16, torch.float16, torch.float32) and q.shape[-1] % 8 == 0 and 0 < q.shape[-1] <= 128
 
 

@@ -124,7 +124,7 @@ def xdit_ring_flash_attn_forward(process_group, q, k, v, softmax_scale, dropout_
     out = None
     lse = None
     final = None
-    # head_dim up to 128 (fp8: 128): every step is one launch that folds its block into the
+    # head_dim up to 128 (fp8: 128 or 64): every step is one launch that folds its block into the
     # accumulator in the kernel's epilogue (same bits as kernel call + update_out_and_lse).
     fused = P > 1 and ops.fused_ring_step_supported(q)
     t = lambda x: None if x is None else x.transpose(1, 2)
