@@ -83,3 +83,35 @@ def test_noalloc_refuses_what_does_not_fit(gpu):
     ops.attn_fwd(q, small_k, small_k, out=out, lse=lse, noalloc=True)
     ref, _ = ops.attn_fwd(q, small_k, small_k)
     assert torch.equal(out, ref)
+
+
+def test_noalloc_call_under_graph_capture(gpu):
+    """The entry point is meant for code under HIP graph capture: once a first call on the device has
+    been made outside capture (it looks up the scratch array's address and sets a kernel attribute),
+    a captured call allocates nothing, and its replays, with eager work of the same entry point in
+    between, give the eager result bit for bit every time."""
+    g = torch.Generator(device=gpu).manual_seed(8)
+    q, k, v = (torch.randn(1, 3, 4608, 128, generator=g, device=gpu).bfloat16() for _ in range(3))
+    q2, k2, v2 = (torch.randn(1, 24, 4608, 128, generator=g, device=gpu).bfloat16() for _ in range(3))
+    assert ops.launch_plan(q, k)["ranges"] > 0
+    out = torch.empty_like(q)
+    lse = torch.empty(1, 3, 4608, device=gpu)
+    want_o, want_l = ops.attn_fwd(q, k, v)
+    ops.attn_fwd(q, k, v, out=out, lse=lse, noalloc=True)   # first call on the device: outside capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.attn_fwd(q, k, v, out=out, lse=lse, noalloc=True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.attn_fwd(q, k, v, out=out, lse=lse, noalloc=True)
+    o2, l2 = torch.empty_like(q2), torch.empty(1, 24, 4608, device=gpu)
+    for replay in range(3):
+        out.zero_(); lse.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_o) and torch.equal(lse, want_l), replay
+        ops.attn_fwd(q2, k2, v2, out=o2, lse=l2, noalloc=True)   # eager work on the same scratch between replays
+        torch.cuda.synchronize()
