@@ -72,7 +72,10 @@ bool mfma16_path(const xdit_attn_args* a) {
 //   time = rate * (KV iterations of the busiest workgroup) * rows * (workgroups sharing its compute unit)
 //          + (segments of that workgroup) * (workgroups sharing ...) * (exposed cost of a segment's prologue and epilogue)
 //          + for a balanced launch: its extra launches, and the partial results a compute unit writes and folds.
-// `plain`: the launch will not be balanced (the ring step, or a call without a workspace).
+// `plain`: the launch will not be balanced (a call without a workspace); `fold_only`: the ring step,
+// whose shared tiles are folded inside the attention kernel (plans of at most 16 parts per tile and
+// 128- or 256-row workgroups, and about 25 us for the fold on top).  fp8 at head_dim 64 is planned
+// with the fp8 constants of head_dim 128.
 // Rate and segment cost depend on what a compute unit holds.  One 4-wavefront workgroup leaves
 // every SIMD a single wavefront with nothing to overlap its softmax with (1.5 times the time per
 // row of 12 wavefronts); two of them hide each other's prologue and epilogue, which a lone 8- or
