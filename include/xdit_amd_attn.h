@@ -177,7 +177,7 @@ typedef struct {
   int32_t rows_per_workgroup;
   int32_t query_tiles;
   int32_t kv_iterations;
-  int64_t workspace_bytes;     /* = xdit_attn_workspace_bytes(args) */
+  int64_t workspace_bytes;     /* = xdit_attn_workspace_bytes(args); with ring_step: what xdit_attn_fwd_accumulate asks for */
   int32_t whole_tiles;
   int32_t ranges;
   int32_t range_len;
@@ -249,8 +249,10 @@ int xdit_lse_merge(const xdit_merge_args* args);
  * (B,S,H,1) accumulator of the legacy ring maps without a copy).  bf16 / fp16 / fp32 inputs with
  * head_dim a multiple of 8 up to 128, fp8 inputs with head_dim 128 or 64; XDIT_ERR_UNSUPPORTED
  * otherwise (use the two calls).
- * args->workspace (optional, as for xdit_attn_fwd: xdit_attn_workspace_bytes of the same arguments
- * suffices) lets the launch be balanced: the parts of the shared query tiles are then folded and
+ * args->workspace (optional, as for xdit_attn_fwd; the size this call asks for is the
+ * workspace_bytes of xdit_attn_launch_plan with ring_step = 1, which can differ from
+ * xdit_attn_workspace_bytes because the ring step is planned on its own; a smaller buffer is
+ * valid, the launch is then not balanced) lets the launch be balanced: the parts of the shared query tiles are then folded and
  * folded on into the accumulator by the attention kernel's own workgroups, and the result still
  * equals xdit_attn_fwd with the same workspace and tuning fields + xdit_lse_merge bit for bit.
  * Replaces, per ring step: the kernel call at ring_flash_attn.py:123-134, update_out_and_lse at

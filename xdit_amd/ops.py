@@ -176,7 +176,15 @@ def _build_attn_plan(q, k, v, softmax_scale, causal, k2, v2, descales, out_dtype
         r.acc_lse_stride = _lib.Strides(acc_lse.stride(0), acc_lse.stride(1), acc_lse.stride(2))
         plan.ring = r
     with _on_device(device):
-        need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
+        if acc is None:
+            need = _lib.lib().xdit_attn_workspace_bytes(ctypes.byref(a))
+        else:
+            # the ring step is planned on its own (its shared tiles are folded inside the kernel): its
+            # launch plan says what it asks for; 0 where it has no plan (the call itself reports why)
+            lp = _lib.LaunchPlan()
+            lp.struct_size = ctypes.sizeof(_lib.LaunchPlan)
+            lp.ring_step = 1
+            need = lp.workspace_bytes if _lib.lib().xdit_attn_launch_plan(ctypes.byref(a), ctypes.byref(lp)) == 0 else 0
     if need < 0:
         _lib.check(need)
     plan.need = need
