@@ -770,6 +770,96 @@ def test_random_problems_vs_oracle(gpu, monkeypatch, seed):
             assert _err(acc_o, mo) <= tol and _err(acc_l, ml) <= 1e-3 and _err(fin, mo) <= tol, what
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(6))
+def test_random_problems_planned_for_few_compute_units(gpu, monkeypatch, seed):
+    """Random small problems launched as if the chip had 3 to 24 compute units (the cu_count field
+    of xdit_attn_args), so that they run in several rounds, with balanced last rounds, ranges taken
+    from the counter, streamed sharing and the fold inside the ring step, in bf16, fp16 and fp8
+    (head_dim 64 and 128) with ragged lengths, a second KV segment and both layouts.  Checked: the
+    oracle's values; the same bits from a second call and from the entry point that allocates
+    nothing (fixed work geometry); the ring step against forward + merge, bit for bit wherever the
+    two launches cut the KV iterations the same way."""
+    import random
+    rnd = random.Random(4000 + seed)
+    g = torch.Generator().manual_seed(100 + seed)
+    seen = {"balanced": 0, "ring_balanced": 0}
+    for case in range(6):
+        kind = rnd.choice(["bf16", "fp16", "fp8", "fp8"])
+        dtype = torch.float16 if kind == "fp16" else torch.bfloat16
+        D = rnd.choice([64, 128]) if kind == "fp8" else 8 * rnd.randint(1, 16)
+        B, H = rnd.randint(1, 2), rnd.randint(1, 6)
+        Sq = rnd.choice([129, 300, 385, 700, 1153])
+        Sk = rnd.choice([65, 1000, 1152, 3000, 9000])
+        Sk2 = rnd.choice([0, 1, 77, 256])
+        if Sk == 9000:   # long shares (ranges from the counter): keep the oracle's work small
+            B, H = 1, min(H, 3)
+        tune = {"rows_per_workgroup": rnd.choice([0, 128, 256, 384]), "balance": rnd.choice([0, 2, 2]),
+                "cu_count": rnd.choice([3, 4, 8, 16, 24]), "streamed": rnd.choice([0, 0, 1])}
+        for name, value in tune.items():
+            monkeypatch.setitem(ops.TUNING, name, value)
+        what = (seed, case, kind, D, B, H, Sq, Sk, Sk2, tune)
+        mk = lambda n: torch.randn(B, H, n, D, generator=g)
+        q, k, v = mk(Sq), mk(Sk), mk(Sk)
+        k2, v2 = (mk(Sk2), mk(Sk2)) if Sk2 else (None, None)
+        lay = lambda t: None if t is None else _layout(t, rnd.choice(["bhsd", "bshd"]), gpu)
+        kw = {}
+        if kind == "fp8":
+            q8, qs = ops.fp8_quant(q.to(gpu))
+            if Sk2:
+                k8, j8, ks = ops.fp8_quant(k.to(gpu), x2=k2.to(gpu))
+                v8, w8, vs = ops.fp8_quant(v.to(gpu), x2=v2.to(gpu))
+            else:
+                (k8, ks), (v8, vs), j8, w8 = ops.fp8_quant(k.to(gpu)), ops.fp8_quant(v.to(gpu)), None, None
+            deq = lambda t, sc: None if t is None else O.dequant(t.cpu(), sc.cpu())
+            qr, kr, vr, k2r, v2r = deq(q8, qs), deq(k8, ks), deq(v8, vs), deq(j8, ks), deq(w8, vs)
+            ins = [t if t is None else lay(t.cpu().view(torch.uint8)).view(torch.float8_e4m3fn) for t in (q8, k8, v8, j8, w8)]
+            kw = dict(q_descale=qs, k_descale=ks, v_descale=vs, out_dtype=dtype)
+            tol_rel, tol_abs = 2.0 ** -4, 6e-2   # one unit in the last place of an e4m3 probability
+        else:
+            qr, kr, vr = q.to(dtype), k.to(dtype), v.to(dtype)
+            k2r, v2r = (k2.to(dtype), v2.to(dtype)) if Sk2 else (None, None)
+            ins = [lay(t) for t in (qr, kr, vr, k2r, v2r)]
+            tol_rel, tol_abs = 2.0 ** -8, 2e-2
+        qd, kd, vd, k2d, v2d = ins
+        kall, vall = (kr, vr) if not Sk2 else (torch.cat([kr, k2r], 2), torch.cat([vr, v2r], 2))
+        ro, rl = O.attn_fwd_ref(qr, kall, vall)
+        o, l = ops.attn_fwd(qd, kd, vd, k2=k2d, v2=v2d, **kw)
+        # outputs here are not averages over many keys and reach 3-4: the bound scales with them
+        assert _err(o, ro) <= max(tol_abs, tol_rel * ro.abs().max().item()) and _err(l, rl) <= 1e-3, what
+        plan = ops.launch_plan(qd, kd, k2=k2d)
+        seen["balanced"] += plan["ranges"] > 0
+        if not tune["streamed"]:
+            o2, l2 = ops.attn_fwd(qd, kd, vd, k2=k2d, v2=v2d, **kw)
+            assert torch.equal(o, o2) and torch.equal(l, l2), what
+            if 0 < plan["workspace_bytes"] <= 32 * 1024 * 1024:
+                o3, l3 = torch.full_like(o, float("nan")), torch.full_like(l, float("nan"))
+                ops.attn_fwd(qd, kd, vd, k2=k2d, v2=v2d, out=o3, lse=l3, noalloc=True, **kw)
+                assert torch.equal(o, o3) and torch.equal(l, l3), what
+        # ring: the block of (k, v) alone, then this call's keys folded on top
+        acc_o = torch.full((B, H, Sq, D), float("nan"), device=gpu)
+        acc_l = torch.full((B, H, Sq), float("nan"), device=gpu)
+        ref_o, ref_l = torch.empty_like(acc_o), torch.empty_like(acc_l)
+        fin = torch.empty(B, H, Sq, D, dtype=dtype, device=gpu)
+        ref_fin = torch.empty_like(fin)
+        ops.attn_fwd_accumulate(qd, kd, vd, acc_o, acc_l, first=True, **kw)
+        bo, bl = ops.attn_fwd(qd, kd, vd, **kw)
+        ops.lse_merge(ref_o, ref_l, bo, bl, first=True)
+        ops.attn_fwd_accumulate(qd, kd, vd, acc_o, acc_l, final_out=fin, k2=k2d, v2=v2d, **kw)
+        ops.lse_merge(ref_o, ref_l, o, l, final_out=ref_fin)
+        r1o, r1l = O.attn_fwd_ref(qr, kr, vr)
+        mo, ml = O.merge_ref(r1o.to(dtype).double(), r1l, ro.to(dtype), rl)
+        assert _err(fin, mo) <= max(tol_abs, 2 * tol_rel * mo.abs().max().item()) and _err(acc_l, ml) <= 1e-3, what
+        ring_plans = [ops.launch_plan(qd, kd, k2=x, ring_step=True) for x in (None, k2d)]
+        seen["ring_balanced"] += ring_plans[1]["ranges"] > 0
+        same_cut = all((a["ranges"] == 0 and b["ranges"] == 0) or
+                       all(a[f] == b[f] for f in ("rows_per_workgroup", "ranges", "range_len", "whole_tiles", "claimers"))
+                       for a, b in zip([ops.launch_plan(qd, kd, k2=x) for x in (None, k2d)], ring_plans))
+        if not tune["streamed"] and same_cut:
+            assert torch.equal(fin, ref_fin) and torch.equal(acc_l, ref_l) and torch.equal(acc_o, ref_o), what
+    assert seen["balanced"] + seen["ring_balanced"] > 0, seen   # the seeds do reach balanced launches
+
+
 # ---------------------------------------------------------------------------- fused ring step
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64),
