@@ -239,6 +239,8 @@ int xdit_lse_merge(const xdit_merge_args* args);
  * into the fp32 accumulator (acc_out, acc_lse) in the kernel's epilogue with the arithmetic of
  * xdit_lse_merge.  The block's rows are rounded to `out_dtype` before the fold, as if they had gone
  * through a block_out tensor, so the result equals xdit_attn_fwd + xdit_lse_merge bit for bit
+ * (when neither launch is balanced, or both cut the KV iterations of their shared query tiles the
+ * same way, which xdit_attn_launch_plan shows; to rounding of the block otherwise)
  * while the block is never written to memory and the accumulator is touched once.
  *   first != 0            initialise the accumulator from this block (acc_out is not read)
  *   args->out  (or NULL)  receives the merged rows in out_dtype: the final step's cast
@@ -252,9 +254,10 @@ int xdit_lse_merge(const xdit_merge_args* args);
  * args->workspace (optional, as for xdit_attn_fwd; the size this call asks for is the
  * workspace_bytes of xdit_attn_launch_plan with ring_step = 1, which can differ from
  * xdit_attn_workspace_bytes because the ring step is planned on its own; a smaller buffer is
- * valid, the launch is then not balanced) lets the launch be balanced: the parts of the shared query tiles are then folded and
- * folded on into the accumulator by the attention kernel's own workgroups, and the result still
- * equals xdit_attn_fwd with the same workspace and tuning fields + xdit_lse_merge bit for bit.
+ * valid, the launch is then not balanced) lets the launch be balanced: the parts of the shared
+ * query tiles are then folded, and folded on into the accumulator, by the attention kernel's own
+ * workgroups, and the result still equals a balanced xdit_attn_fwd with the same ranges +
+ * xdit_lse_merge bit for bit.
  * Replaces, per ring step: the kernel call at ring_flash_attn.py:123-134, update_out_and_lse at
  * :138 and, on the last step, the cast at :145.
  */
