@@ -468,6 +468,15 @@ def main():
                                        "gbs": round(qw.numel() * 5.0 / st["ms"] / 1e6, 1),
                                        "frac_hbm_peak": round(qw.numel() * 5.0 / st["ms"] / 1e6 / PEAK_HBM_GBS, 4)}
         del qw, kw, vw, q8, k8, v8
+        # head_dim 64 (what the hybrid schedule hands the fp8 backend for SD3 and CogVideoX), fp8 beside bf16
+        for name, (Bs, Hs, Ss) in (("sd3_1024_d64", (2, 24, 4250)), ("cogvideox_d64", (2, 48, 17776))):
+            qs, ks, vs = make_inputs(Bs, Hs, Ss, 64, 1006, dev)
+            (q8, qd), (k8, kd), (v8, vd) = (ops.fp8_quant(t) for t in (qs, ks, vs))
+            fl = attn_flops(Bs, Hs, Ss, Ss, 64)
+            n = 5 if Ss > 8192 else 40
+            also[name + "_fp8"] = with_rate(time_each(lambda: ops.attn_fwd(q8, k8, v8, q_descale=qd, k_descale=kd, v_descale=vd), n, 3), fl, PEAK_FP8_TFLOPS)
+            also[name + "_bf16"] = with_rate(time_each(lambda: ops.attn_fwd(qs, ks, vs), n, 3), fl, PEAK_BF16_TFLOPS)
+            del qs, ks, vs, q8, k8, v8
         # pre-attention prologue (per-head RMSNorm + rotary embedding + BSHD -> BHSD), bf16:
         # bytes per call = 4*N*D (read + write) + 8*S*D (cos and sin rows, read once)
         from xdit_amd import prologue
